@@ -4,11 +4,11 @@ from . import errors
 from .errors import (BackendError, CacheError, ConfigError, HerbertError, ModelLoadError,
                      RequestError)
 from . import config, weights, cache, parts, models
-from .config import ModasunConfig, Qwen3Config, VipalornConfig, load_config, register_architecture
+from .config import MefatarConfig, ModasunConfig, Qwen3Config, VipalornConfig, load_config, register_architecture
 from .engine import Engine, StepEntry
 from .sampling import SamplingParams
 from .api import generate, load, write_random_model
 
 __all__ = ["BackendError", "CacheError", "ConfigError", "Engine", "HerbertError", "ModelLoadError",
-           "ModasunConfig", "Qwen3Config", "RequestError", "SamplingParams", "StepEntry", "VipalornConfig", "generate", "load",
+           "MefatarConfig", "ModasunConfig", "Qwen3Config", "RequestError", "SamplingParams", "StepEntry", "VipalornConfig", "generate", "load",
            "load_config", "register_architecture", "write_random_model"]

@@ -5,6 +5,7 @@ from .registry import (Architecture, ChatFormat, load_config, register_architect
 from .qwen3 import Qwen3Config
 from .vipalorn import VipalornConfig
 from .modasun import ModasunConfig
+from .mefatar import MefatarConfig
 
-__all__ = ["Architecture", "ChatFormat", "ModasunConfig", "Qwen3Config", "VipalornConfig", "load_config", "read_config_json",
+__all__ = ["Architecture", "ChatFormat", "MefatarConfig", "ModasunConfig", "Qwen3Config", "VipalornConfig", "load_config", "read_config_json",
            "register_architecture", "registered_architectures", "resolve_architecture"]

@@ -9,7 +9,9 @@
 // (crates/backends/backend_common/src/generic_attention/decode.rs:126), causal by count
 // (crates/backends/backend_common/src/generic_attention/prefill/kernel_f32.rs:65-67), online softmax and
 // sum of p v (kernel_f32.rs:83-110; decoding: crates/backends/backend_common/src/attention_common.rs:141-178),
-// all float32. The window is not in the reference, which never reads those keys.
+// all float32. The window is not in the reference, which never reads those keys. Nor is the sink: with
+// `sinks` [nq] given, the softmax's denominator of head h also holds exp(sinks[h]), a score without a key
+// and a value, unscaled, counted once (the running maximum starts there and the running sum at one).
 #include "common.h"
 #include <math.h>
 
@@ -24,7 +26,8 @@ attention_plain_kernel(const TQ* __restrict__ q, const TC* __restrict__ k_cache,
                        const TC* __restrict__ v_cache, TO* __restrict__ out,
                        const int* __restrict__ positions, const int* __restrict__ seq_of,
                        const int* __restrict__ slots, const int* __restrict__ page_table, int max_pages,
-                       int page_size, int nq, int nkv, int hd, float scale, int window) {
+                       int page_size, int nq, int nkv, int hd, float scale, int window,
+                       const float* __restrict__ sinks) {
     __shared__ float qs[HB_MAX_HEAD_DIM];
     __shared__ float ps[HB_WAVE];
     const int t = blockIdx.x;
@@ -42,6 +45,7 @@ attention_plain_kernel(const TQ* __restrict__ q, const TC* __restrict__ k_cache,
     const int hi = pos + 1;
     const int lo = (window > 0 && hi > window) ? hi - window : 0;
     float m = -INFINITY, l = 0.f;
+    if (sinks) m = sinks[h], l = 1.0f;
     float acc[ACC_REGS];
 #pragma unroll
     for (int i = 0; i < ACC_REGS; ++i) acc[i] = 0.f;
@@ -97,7 +101,8 @@ attention_plain_kernel(const TQ* __restrict__ q, const TC* __restrict__ k_cache,
 extern "C" int hb_attention_plain(const void* q, const void* k_cache, const void* v_cache, void* out,
                                   int dtype, const int* positions, const int* seq_of, const int* slots,
                                   const int* page_table, int max_pages, int page_size, int T, int nq,
-                                  int nkv, int hd, float scale, int window, hipStream_t stream) {
+                                  int nkv, int hd, float scale, int window, const float* sinks,
+                                  hipStream_t stream) {
     HB_REQUIRE(T > 0 && nq > 0 && nkv > 0, "attention: empty input");
     HB_REQUIRE(nq % nkv == 0, "attention: %d query heads not divisible by %d kv heads", nq, nkv);
     HB_REQUIRE(hd > 0 && hd <= HB_MAX_HEAD_DIM, "attention: head_dim %d not in 1..%d", hd,
@@ -108,11 +113,11 @@ extern "C" int hb_attention_plain(const void* q, const void* k_cache, const void
     if (dtype == HB_F32)
         attention_plain_kernel<float, float, float><<<grid, HB_WAVE, 0, stream>>>(
             (const float*)q, (const float*)k_cache, (const float*)v_cache, (float*)out, positions, seq_of,
-            slots, page_table, max_pages, page_size, nq, nkv, hd, scale, window);
+            slots, page_table, max_pages, page_size, nq, nkv, hd, scale, window, sinks);
     else if (dtype == HB_BF16)
         attention_plain_kernel<bf16, bf16, bf16><<<grid, HB_WAVE, 0, stream>>>(
             (const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, positions, seq_of,
-            slots, page_table, max_pages, page_size, nq, nkv, hd, scale, window);
+            slots, page_table, max_pages, page_size, nq, nkv, hd, scale, window, sinks);
     else
         HB_REQUIRE(false, "attention: unknown dtype %d", dtype);
     HB_CHECK_LAUNCH("attention_plain");

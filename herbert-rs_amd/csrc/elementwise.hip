@@ -429,9 +429,16 @@ extern "C" int hb_qk_norm_rope_write(const float* qkv, int ld_qkv, const float* 
     return 0;
 }
 
-// ------------------------------------------------------------------- SwiGLU
-// act[t, i] = silu(gu[t, i]) * gu[t, I + i], silu(g) = g / (1 + exp(-g)).
-template <class TOut>
+// ------------------------------------------------------------------- gated linear units
+// act[t, i] = f(gu[t, i]) * gu[t, I + i] with f = silu, g / (1 + exp(-g)), or the tanh form of gelu,
+// 0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3))).
+#define HB_ACT_SILU 0
+#define HB_ACT_GELU_TANH 1
+__device__ __forceinline__ float hb_gelu_tanh(float z) {
+    return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+template <class TOut, int ACT>
 __global__ void swiglu_kernel(const float* __restrict__ gu, TOut* __restrict__ act, int I, size_t total) {
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total) return;
@@ -439,19 +446,23 @@ __global__ void swiglu_kernel(const float* __restrict__ gu, TOut* __restrict__ a
     const int i = (int)(idx - t * I);
     const float g = gu[t * 2 * I + i];
     const float u = gu[t * 2 * I + I + i];
-    act[idx] = hb_from_float<TOut>(g / (1.0f + expf(-g)) * u);
+    const float f = ACT == HB_ACT_GELU_TANH ? hb_gelu_tanh(g) : g / (1.0f + expf(-g));
+    act[idx] = hb_from_float<TOut>(f * u);
 }
 
-extern "C" int hb_swiglu(const float* gu, void* act, int act_dtype, int T, int I, hipStream_t stream) {
+extern "C" int hb_swiglu(const float* gu, void* act, int act_dtype, int T, int I, int activation, hipStream_t stream) {
     HB_REQUIRE(T > 0 && I > 0, "swiglu: empty input");
+    HB_REQUIRE(activation == HB_ACT_SILU || activation == HB_ACT_GELU_TANH, "swiglu: unknown activation %d", activation);
+    HB_REQUIRE(act_dtype == HB_F32 || act_dtype == HB_BF16, "swiglu: unknown output dtype %d", act_dtype);
     const size_t total = (size_t)T * I;
     const unsigned blocks = (unsigned)((total + 255) / 256);
-    if (act_dtype == HB_F32)
-        swiglu_kernel<float><<<blocks, 256, 0, stream>>>(gu, (float*)act, I, total);
-    else if (act_dtype == HB_BF16)
-        swiglu_kernel<bf16><<<blocks, 256, 0, stream>>>(gu, (bf16*)act, I, total);
-    else
-        HB_REQUIRE(false, "swiglu: unknown output dtype %d", act_dtype);
+    if (act_dtype == HB_F32) {
+        if (activation == HB_ACT_SILU) swiglu_kernel<float, HB_ACT_SILU><<<blocks, 256, 0, stream>>>(gu, (float*)act, I, total);
+        else swiglu_kernel<float, HB_ACT_GELU_TANH><<<blocks, 256, 0, stream>>>(gu, (float*)act, I, total);
+    } else {
+        if (activation == HB_ACT_SILU) swiglu_kernel<bf16, HB_ACT_SILU><<<blocks, 256, 0, stream>>>(gu, (bf16*)act, I, total);
+        else swiglu_kernel<bf16, HB_ACT_GELU_TANH><<<blocks, 256, 0, stream>>>(gu, (bf16*)act, I, total);
+    }
     HB_CHECK_LAUNCH("swiglu");
     return 0;
 }
@@ -672,5 +683,234 @@ extern "C" int hb_relu_squared(const float* z, void* act, int act_dtype, size_t 
     else
         HB_REQUIRE(false, "relu_squared: unknown output dtype %d", act_dtype);
     HB_CHECK_LAUNCH("relu_squared");
+    return 0;
+}
+
+// ------------------------------------------- RMSNorm that first takes a scaled sum on
+// x[r, :] += ls * delta[r, :] (ls a factor a column), written back to x, then y[r, :] = x / rms(x) * w: the
+// one kernel between two branches of a pre-norm layer whose branches are scaled channel by channel.
+// y null: only the sum (after the last layer).
+template <class TOut>
+__global__ void rmsnorm_scaled_sum_kernel(float* x, const float* __restrict__ delta, const float* __restrict__ ls,
+                                          const float* __restrict__ w, TOut* y, int H, float eps) {
+    __shared__ float red[16];
+    const size_t row = (size_t)blockIdx.x * H;
+    float* in = x + row;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        const float v = fmaf(ls[i], delta[row + i], in[i]);
+        in[i] = v;
+        ss += v * v;
+    }
+    if (y == nullptr) return;
+    ss = hb_block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+    TOut* out = y + row;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = hb_from_float<TOut>(in[i] * inv * w[i]);
+}
+
+extern "C" int hb_rmsnorm_scaled_sum(float* x, const float* delta, const float* ls, const float* w, void* y,
+                                     int y_dtype, int R, int H, float eps, hipStream_t stream) {
+    HB_REQUIRE(R > 0 && H > 0, "rmsnorm: empty input (R=%d, H=%d)", R, H);
+    HB_REQUIRE(delta != nullptr && ls != nullptr, "rmsnorm: a scaled sum needs its rows and its factors");
+    HB_REQUIRE(y == nullptr || w != nullptr, "rmsnorm: a norm needs its weight");
+    HB_REQUIRE(y_dtype == HB_F32 || y_dtype == HB_BF16, "rmsnorm: unknown output dtype %d", y_dtype);
+    const int threads = H >= 1024 ? 256 : H >= 256 ? 128 : 64;
+    if (y_dtype == HB_F32)
+        rmsnorm_scaled_sum_kernel<float><<<R, threads, 0, stream>>>(x, delta, ls, w, (float*)y, H, eps);
+    else
+        rmsnorm_scaled_sum_kernel<bf16><<<R, threads, 0, stream>>>(x, delta, ls, w, (bf16*)y, H, eps);
+    HB_CHECK_LAUNCH("rmsnorm_scaled_sum");
+    return 0;
+}
+
+// ------------------------------------------- two rows normed and weighed into one
+// out[r, :] (+)= ca * a[r, :] / rms(a[r]) * wa + cb * b[r, :] / rms(b[r]) * wb: the outputs of two mixers
+// that ran side by side, each normed over the model's width, joined. float32 throughout.
+template <bool ACCUM>
+__global__ void normed_pair_kernel(const float* __restrict__ a, const float* __restrict__ wa, float ca,
+                                   const float* __restrict__ b, const float* __restrict__ wb, float cb,
+                                   float* out, int H, float eps) {
+    __shared__ float red[16];
+    const size_t row = (size_t)blockIdx.x * H;
+    float sa = 0.f, sb = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        const float va = a[row + i], vb = b[row + i];
+        sa += va * va;
+        sb += vb * vb;
+    }
+    sa = hb_block_sum(sa, red);
+    sb = hb_block_sum(sb, red);
+    const float ia = ca / sqrtf(sa / (float)H + eps), ib = cb / sqrtf(sb / (float)H + eps);
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        const float v = a[row + i] * ia * wa[i] + b[row + i] * ib * wb[i];
+        out[row + i] = ACCUM ? out[row + i] + v : v;
+    }
+}
+
+extern "C" int hb_normed_pair(const float* a, const float* wa, float ca, const float* b, const float* wb, float cb,
+                              float* out, int R, int H, float eps, int accumulate, hipStream_t stream) {
+    HB_REQUIRE(R > 0 && H > 0, "normed pair: empty input (R=%d, H=%d)", R, H);
+    const int threads = H >= 1024 ? 256 : H >= 256 ? 128 : 64;
+    if (accumulate)
+        normed_pair_kernel<true><<<R, threads, 0, stream>>>(a, wa, ca, b, wb, cb, out, H, eps);
+    else
+        normed_pair_kernel<false><<<R, threads, 0, stream>>>(a, wa, ca, b, wb, cb, out, H, eps);
+    HB_CHECK_LAUNCH("normed_pair");
+    return 0;
+}
+
+// ------------------------------------------- filter along time + norm over the whole projection
+//                                             + rotation of neighbouring pairs + cache write
+// A row of the fused projection holds [nq x dim queries | nkv x dim keys | nkv x vdim values] in its first
+// C columns. One workgroup a token:
+//   filter (taps [C, K], K >= 1; null: none): y[c] = sum_j taps[c, j] * in[t - (K - 1) + j, c], the inputs
+//     before the step's first row from the slot's state [K - 1, C] (zeros in a fresh slot); the state is
+//     moved on by a kernel of its own afterwards (hb_filter_state in the module of the recurrent mixers);
+//   norm (weights null: none): all queries of the token are divided by their common root mean square and
+//     multiplied by q_norm_w [nq x dim], the keys likewise with k_norm_w [nkv x dim];
+//   rotation (rates null: none): entries 2i and 2i + 1 of the first rot_dims of every query and key head turn
+//     by position x rates[i]; rates are float64 and so are the angle, its sine and its cosine;
+//   q_out [T, nq x hd], key pages [page, kv head, token, hd], value pages [page, kv head, hd, token]: heads
+//     are kept at size hd >= max(dim, vdim), the entries beyond a head's own size are zeros.
+template <class TQ, class TC>
+__global__ void __launch_bounds__(256)
+filter_norm_rotate_write_kernel(const float* __restrict__ proj, int ld, const float* __restrict__ taps, int K,
+                                const float* __restrict__ filter_state, const float* __restrict__ q_norm_w,
+                                const float* __restrict__ k_norm_w, const double* __restrict__ rates, int rot_dims,
+                                const int* __restrict__ positions, const int* __restrict__ seq_of,
+                                const int* __restrict__ seq_starts, const int* __restrict__ slots,
+                                const int* __restrict__ page_table, int max_pages, int page_size,
+                                TQ* __restrict__ q_out, TC* __restrict__ k_cache, TC* __restrict__ v_cache, int nq,
+                                int nkv, int dim, int vdim, int hd, float eps) {
+    extern __shared__ float filtered[];           // [C] the token's channels, then [rot_dims] cosines and sines
+    __shared__ float red[16];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const int QD = nq * dim, KD = nkv * dim, C = QD + KD + nkv * vdim;
+    float* cs = filtered + C;
+    const int seq = seq_of[t];
+    const int first = seq_starts[seq];
+    const int at = t - first;
+    const int slot = slots[seq];
+    const int pos = positions[t];
+    const float* state = filter_state + (size_t)slot * (K > 1 ? K - 1 : 1) * C;
+    float sq = 0.f, sk = 0.f;
+    for (int c = tid; c < C; c += 256) {
+        float y;
+        if (taps == nullptr) {
+            y = proj[(size_t)t * ld + c];
+        } else {
+            y = 0.f;
+            for (int j = 0; j < K; ++j) {
+                const int s = at - (K - 1) + j;
+                const float v = s >= 0 ? proj[(size_t)(first + s) * ld + c] : state[(size_t)(K - 1 + s) * C + c];
+                y = fmaf(taps[(size_t)c * K + j], v, y);
+            }
+        }
+        filtered[c] = y;
+        if (c < QD) sq = fmaf(y, y, sq);
+        else if (c < QD + KD) sk = fmaf(y, y, sk);
+    }
+    if (rates != nullptr) {
+        for (int i = tid; i < rot_dims / 2; i += 256) {
+            double s, c;
+            sincos((double)pos * rates[i], &s, &c);
+            cs[2 * i] = (float)c;
+            cs[2 * i + 1] = (float)s;
+        }
+    }
+    sq = hb_block_sum(sq, red);           // (its barriers also publish `filtered` and the angles)
+    sk = hb_block_sum(sk, red);
+    const float inv_q = q_norm_w ? 1.0f / sqrtf(sq / (float)QD + eps) : 1.0f;
+    const float inv_k = k_norm_w ? 1.0f / sqrtf(sk / (float)KD + eps) : 1.0f;
+    const int rd = rates != nullptr ? rot_dims : 0;
+    // one entry of a query or key head after norm and rotation; c0: the head's first channel
+    auto turned = [&](int c0, int d, const float* w, float inv) {
+        if (d >= dim) return 0.f;
+        auto normed = [&](int e) { return w ? filtered[c0 + e] * inv * w[c0 + e] : filtered[c0 + e]; };
+        if (d >= rd) return normed(d);
+        const int i = d >> 1;
+        const float u = normed(2 * i), v = normed(2 * i + 1);
+        const float co = cs[2 * i], si = cs[2 * i + 1];
+        return (d & 1) ? v * co + u * si : u * co - v * si;
+    };
+    for (int idx = tid; idx < nq * hd; idx += 256) {
+        const int h = idx / hd, d = idx - h * hd;
+        q_out[(size_t)t * nq * hd + idx] = hb_from_float<TQ>(turned(h * dim, d, q_norm_w, inv_q));
+    }
+    const int page = page_table[(size_t)slot * max_pages + pos / page_size];
+    const int in_page = pos % page_size;
+    for (int idx = tid; idx < nkv * hd; idx += 256) {
+        const int g = idx / hd, d = idx - g * hd;
+        const float* kw = k_norm_w ? k_norm_w - QD : nullptr;       // (indexed by the channel within the row)
+        const size_t base = ((size_t)page * nkv + g) * page_size * hd;
+        k_cache[base + (size_t)in_page * hd + d] = hb_from_float<TC>(turned(QD + g * dim, d, kw, inv_k));
+        const float v = d < vdim ? filtered[QD + KD + g * vdim + d] : 0.f;
+        v_cache[base + (size_t)d * page_size + in_page] = hb_from_float<TC>(v);
+    }
+}
+
+extern "C" int hb_filter_norm_rotate_write(const float* proj, int ld, const float* taps, int K, const float* filter_state,
+                                           const float* q_norm_w, const float* k_norm_w, const double* rates,
+                                           int rot_dims, const int* positions, const int* seq_of,
+                                           const int* seq_starts, const int* slots, const int* page_table,
+                                           int max_pages, int page_size, void* q_out, void* k_cache, void* v_cache,
+                                           int dtype, int T, int nq, int nkv, int dim, int vdim, int hd, float eps,
+                                           hipStream_t stream) {
+    HB_REQUIRE(T > 0 && nq > 0 && nkv > 0 && dim > 0 && vdim > 0, "filtered attention: empty input");
+    HB_REQUIRE(hd >= dim && hd >= vdim, "filtered attention: heads kept at %d cannot hold %d and %d", hd, dim, vdim);
+    const long long C = (long long)(nq + nkv) * dim + (long long)nkv * vdim;
+    HB_REQUIRE(ld >= C, "filtered attention: rows of %d do not hold %lld channels", ld, C);
+    HB_REQUIRE(taps == nullptr || (K >= 1 && K <= 16), "filtered attention: %d taps, the kernel takes 1 to 16", K);
+    HB_REQUIRE(taps == nullptr || K == 1 || filter_state != nullptr, "filtered attention: a filter needs its state");
+    HB_REQUIRE(rates == nullptr || (rot_dims > 0 && rot_dims % 2 == 0 && rot_dims <= dim),
+               "filtered attention: %d rotated entries of heads of %d", rot_dims, dim);
+    const size_t lds = ((size_t)C + (rates ? rot_dims : 0)) * sizeof(float);
+    HB_REQUIRE(lds <= 60 * 1024, "filtered attention: %lld channels a token do not fit the kernel's LDS", C);
+    if (taps == nullptr) K = 0;
+    if (dtype == HB_F32)
+        filter_norm_rotate_write_kernel<float, float><<<T, 256, lds, stream>>>(
+            proj, ld, taps, K, filter_state, q_norm_w, k_norm_w, rates, rot_dims, positions, seq_of, seq_starts, slots,
+            page_table, max_pages, page_size, (float*)q_out, (float*)k_cache, (float*)v_cache, nq, nkv, dim, vdim, hd, eps);
+    else if (dtype == HB_BF16)
+        filter_norm_rotate_write_kernel<bf16, bf16><<<T, 256, lds, stream>>>(
+            proj, ld, taps, K, filter_state, q_norm_w, k_norm_w, rates, rot_dims, positions, seq_of, seq_starts, slots,
+            page_table, max_pages, page_size, (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, nq, nkv, dim, vdim, hd, eps);
+    else
+        HB_REQUIRE(false, "filtered attention: unknown dtype %d", dtype);
+    HB_CHECK_LAUNCH("filter_norm_rotate_write");
+    return 0;
+}
+
+// ------------------------------------------- a gate on the heads' outputs
+// out[t, h x vdim + d] = attn[t, h x hd + d] * sigmoid(gate[t, g_off + h x vdim + d]) for d < vdim: the heads'
+// outputs, kept at size hd, leave at their own size, each entry times a gate of its own (gate_rows null: none).
+template <class TIn, class TOut>
+__global__ void gate_heads_kernel(const TIn* __restrict__ attn, const float* __restrict__ gate_rows, int ld, int g_off,
+                                  TOut* __restrict__ out, int nq, int hd, int vdim, size_t total) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int W = nq * vdim;
+    const size_t t = idx / W;
+    const int c = (int)(idx - t * W);
+    const int h = c / vdim, d = c - h * vdim;
+    float v = hb_to_float(attn[(t * nq + h) * hd + d]);
+    if (gate_rows) v *= 1.0f / (1.0f + expf(-gate_rows[t * ld + g_off + c]));
+    out[idx] = hb_from_float<TOut>(v);
+}
+
+extern "C" int hb_gate_heads(const void* attn, int dtype, const float* gate_rows, int ld, int g_off, void* out, int T,
+                             int nq, int hd, int vdim, hipStream_t stream) {
+    HB_REQUIRE(T > 0 && nq > 0 && vdim > 0 && hd >= vdim, "gate: empty input or heads of %d kept at %d", vdim, hd);
+    HB_REQUIRE(gate_rows == nullptr || (g_off >= 0 && g_off + nq * vdim <= ld), "gate: its columns lie outside the rows");
+    const size_t total = (size_t)T * nq * vdim;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    if (dtype == HB_F32)
+        gate_heads_kernel<float, float><<<blocks, 256, 0, stream>>>((const float*)attn, gate_rows, ld, g_off, (float*)out, nq, hd, vdim, total);
+    else if (dtype == HB_BF16)
+        gate_heads_kernel<bf16, bf16><<<blocks, 256, 0, stream>>>((const bf16*)attn, gate_rows, ld, g_off, (bf16*)out, nq, hd, vdim, total);
+    else
+        HB_REQUIRE(false, "gate: unknown dtype %d", dtype);
+    HB_CHECK_LAUNCH("gate_heads");
     return 0;
 }

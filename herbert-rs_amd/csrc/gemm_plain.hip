@@ -18,15 +18,21 @@ HB_MODULE_ERROR_SLOT()
 
 // What a product may do to a sum before it stores it: nothing (rate null), or turn the pre-activation of a
 // decay into the decay itself, exp(-exp(rate[n / D]) * softplus(sum + bias[n])) for column n (float32; the
-// arithmetic of hb_channel_decay, which does the same to rows that lie in memory).
+// arithmetic of hb_channel_decay, which does the same to rows that lie in memory). A decay of the other kind
+// (rate == bias, the mark of it): sigmoid(sum + bias[n])^root = exp(-root * softplus(-(sum + bias[n]))).
 struct DecayEpilogue {
     const float* rate;
     const float* bias;
     int D;
+    float root;
 };
 
 __device__ __forceinline__ float decay_of(const DecayEpilogue& ep, float sum, int n) {
     const float a = sum + ep.bias[n];
+    if (ep.rate == ep.bias) {
+        const float softplus = -a > 20.f ? -a : log1pf(expf(-a));
+        return expf(-ep.root * softplus);
+    }
     const float softplus = a > 20.f ? a : log1pf(expf(a));
     return expf(-expf(ep.rate[n / ep.D]) * softplus);
 }
@@ -103,7 +109,7 @@ gemm_plain_kernel(const TA* __restrict__ A, const TW* __restrict__ W, TC* __rest
 template <class TA, class TW, class TC>
 static void launch(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
                    int accumulate, hipStream_t stream, int batch = 1, size_t batch_a = 0, size_t batch_w = 0,
-                   size_t batch_c = 0, DecayEpilogue ep = DecayEpilogue{nullptr, nullptr, 1}) {
+                   size_t batch_c = 0, DecayEpilogue ep = DecayEpilogue{nullptr, nullptr, 1, 0.f}) {
     dim3 grid((N + TILE_N - 1) / TILE_N, (M + TILE_M - 1) / TILE_M, batch);
     if (accumulate)
         gemm_plain_kernel<TA, TW, TC, true><<<grid, 256, 0, stream>>>(
@@ -209,16 +215,18 @@ extern "C" int hb_gemm_plain(const void* A, int a_dtype, const void* W, int w_dt
 
 // The same product for callers whose k is short (a narrow middle): few rows take the kernel made for them.
 // A_log [N / D] and dt_bias [N], both or neither: the sums are a decay's pre-activations, and what is stored is
-// the decay a column (float32 in and out, no accumulation).
+// the decay a column (float32 in and out, no accumulation). A_log == dt_bias: the decay is
+// sigmoid(sum + dt_bias[n])^root instead.
 extern "C" int hb_gemm_plain_short_k(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype,
                                      int M, int N, int K, int lda, int ldw, int ldc, int accumulate,
-                                     const float* A_log, const float* dt_bias, int D, hipStream_t stream) {
+                                     const float* A_log, const float* dt_bias, int D, float root,
+                                     hipStream_t stream) {
     HB_REQUIRE(M > 0 && N > 0 && K > 0, "gemm: empty problem (M=%d, N=%d, K=%d)", M, N, K);
     HB_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gemm: a row stride is smaller than its row");
     HB_REQUIRE((A_log == nullptr) == (dt_bias == nullptr), "gemm: a decay needs its rate and its bias");
     HB_REQUIRE(!A_log || (D > 0 && N % D == 0 && c_dtype == 0 && !accumulate),
                "gemm: a decay is float32, stored and not added, %d columns in heads of %d", N, D);
-    const DecayEpilogue ep{A_log, dt_bias, A_log ? D : 1};
+    const DecayEpilogue ep{A_log, dt_bias, A_log ? D : 1, root};
     if (few_rows_takes(A, a_dtype, W, w_dtype, c_dtype, M, K, lda, ldw, accumulate)) {
         gemm_few_rows_kernel<<<dim3((N + 15) / 16, (M + FEW_ROWS_M - 1) / FEW_ROWS_M), HB_WAVE, 0, stream>>>(
             (const float*)A, (const bf16*)W, (float*)C, M, N, K, lda, ldw, ldc, ep);

@@ -59,18 +59,20 @@ conv_silu_kernel(const float* __restrict__ proj, int ld, const float* __restrict
 
 // The state after the step: the last K - 1 inputs of each sequence, from the step's rows where it
 // brought that many, else the old state moved up. One thread a (sequence, channel).
+// (bias [C] or null: the inputs are the rows plus a bias a channel, and the state holds them with it)
 __global__ void conv_state_kernel(const float* __restrict__ proj, int ld, float* __restrict__ conv_state,
                                   const int* __restrict__ seq_starts, const int* __restrict__ slots, int C,
-                                  int K) {
+                                  int K, const float* __restrict__ bias) {
     const int seq = blockIdx.x;
     const int c = blockIdx.y * blockDim.x + threadIdx.x;
     if (c >= C) return;
     const int first = seq_starts[seq], n = seq_starts[seq + 1] - first;
     float* state = conv_state + (size_t)slots[seq] * (K - 1) * C;
+    const float b = bias ? bias[c] : 0.f;
     float keep[HB_MAX_TAPS];
     for (int i = 0; i < K - 1; ++i) {
         const int s = n - (K - 1) + i;
-        keep[i] = s >= 0 ? proj[(size_t)(first + s) * ld + c] : state[(size_t)(i + n) * C + c];
+        keep[i] = s >= 0 ? proj[(size_t)(first + s) * ld + c] + b : state[(size_t)(i + n) * C + c];
     }
     for (int i = 0; i < K - 1; ++i) state[(size_t)i * C + c] = keep[i];
 }
@@ -88,9 +90,125 @@ extern "C" int hb_conv_silu(const float* proj, int ld, const float* taps, float*
         unit_eps, plain_dim);
     HB_CHECK_LAUNCH("conv_silu");
     if (K > 1) {
-        conv_state_kernel<<<dim3(B, (C + 255) / 256), 256, 0, stream>>>(proj, ld, conv_state, seq_starts, slots, C, K);
+        conv_state_kernel<<<dim3(B, (C + 255) / 256), 256, 0, stream>>>(proj, ld, conv_state, seq_starts, slots, C, K, nullptr);
         HB_CHECK_LAUNCH("conv_state");
     }
+    return 0;
+}
+
+// The state of a filter alone, for mixers that filter in a kernel of their own: after a step, the last K - 1
+// inputs (the first C columns of proj's rows, plus bias [C] if given) of each sequence.
+extern "C" int hb_filter_state(const float* proj, int ld, float* conv_state, const int* seq_starts, const int* slots,
+                               int B, int C, int K, const float* bias, hipStream_t stream) {
+    HB_REQUIRE(B > 0 && C > 0 && ld >= C && B <= 65535, "filter state: empty input or too many sequences");
+    HB_REQUIRE(K >= 1 && K <= HB_MAX_TAPS, "filter state: %d taps, the kernel takes 1 to %d", K, HB_MAX_TAPS);
+    if (K == 1) return 0;
+    conv_state_kernel<<<dim3(B, (C + 255) / 256), 256, 0, stream>>>(proj, ld, conv_state, seq_starts, slots, C, K, bias);
+    HB_CHECK_LAUNCH("filter_state");
+    return 0;
+}
+
+// ------------------------------------------------------------------ real-gated linear recurrent unit
+// Two branches of W channels from one projection's rows [x | y] (float32, ld apart):
+//   u[t, c] = fb[c] + sum_j taps[c, j] * (x[t - (K - 1) + j, c] + bx[c])     (nothing before a sequence's start; the
+//             inputs before the step's first row come from the slot's state [K - 1, W], which holds them with bx)
+//   g[t, c] = gelu_tanh(y[t, c] + by[c])
+// out rows are [u | g], float32. One thread a (token, channel).
+__device__ __forceinline__ float lru_gelu_tanh(float z) {
+    return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+__global__ void lru_inputs_kernel(const float* __restrict__ proj, int ld, const float* __restrict__ bx,
+                                  const float* __restrict__ by, const float* __restrict__ taps,
+                                  const float* __restrict__ fb, const float* __restrict__ conv_state,
+                                  const int* __restrict__ seq_of, const int* __restrict__ seq_starts,
+                                  const int* __restrict__ slots, float* __restrict__ out, int W, int K) {
+    const int t = blockIdx.x;
+    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= W) return;
+    const int seq = seq_of[t];
+    const int first = seq_starts[seq];
+    const int at = t - first;
+    const float* state = conv_state + (size_t)slots[seq] * (K > 1 ? K - 1 : 1) * W;
+    const float b = bx[c];
+    float acc = fb ? fb[c] : 0.f;
+    for (int j = 0; j < K; ++j) {
+        const int s = at - (K - 1) + j;
+        const float v = s >= 0 ? proj[(size_t)(first + s) * ld + c] + b : state[(size_t)(K - 1 + s) * W + c];
+        acc = fmaf(taps[(size_t)c * K + j], v, acc);
+    }
+    out[(size_t)t * 2 * W + c] = acc;
+    out[(size_t)t * 2 * W + W + c] = lru_gelu_tanh(proj[(size_t)t * ld + W + c] + by[c]);
+}
+
+extern "C" int hb_lru_inputs(const float* proj, int ld, const float* bx, const float* by, const float* taps,
+                             const float* fb, float* conv_state, const int* seq_of, const int* seq_starts,
+                             const int* slots, float* out, int T, int B, int W, int K, hipStream_t stream) {
+    HB_REQUIRE(T > 0 && B > 0 && W > 0 && ld >= 2 * W, "recurrent unit: empty input or rows of %d for 2 x %d channels", ld, W);
+    HB_REQUIRE(K >= 1 && K <= HB_MAX_TAPS, "recurrent unit: %d taps, the kernel takes 1 to %d", K, HB_MAX_TAPS);
+    HB_REQUIRE((W + 255) / 256 <= 65535 && B <= 65535, "recurrent unit: too many channels or sequences for the grid");
+    lru_inputs_kernel<<<dim3(T, (W + 255) / 256), 256, 0, stream>>>(proj, ld, bx, by, taps, fb, conv_state, seq_of,
+                                                                    seq_starts, slots, out, W, K);
+    HB_CHECK_LAUNCH("lru_inputs");
+    if (K > 1) {
+        conv_state_kernel<<<dim3(B, (W + 255) / 256), 256, 0, stream>>>(proj, ld, conv_state, seq_starts, slots, W, K, bx);
+        HB_CHECK_LAUNCH("lru_filter_state");
+    }
+    return 0;
+}
+
+// The recurrence itself, channel by channel:
+//   r = sigmoid(r_pre[t, c] + rb[c]);  i = sigmoid(i_pre[t, c] + ib[c])
+//       (gates rows are float32 [block 0: r, i | block 1: r, i | ...], blocks of bw channels, as a product a block
+//        of the block's u with the block's two stacked matrices leaves them)
+//   a = exp(-rate * r * softplus(lam[c]));  S <- a S + sqrt(1 - a^2) * i * u[t, c];  y[t, c] = S * g[t, c]
+// with S from the slot's state [W] (zero in a fresh slot; the first token is no special case) and u, g the
+// rows that lru_inputs_kernel left. 1 - a^2 is taken as -expm1(2 ln a), which keeps its digits where a is
+// near one. One thread a (sequence, channel) walks the sequence's tokens; the loads of a token do not wait
+// for the chain, which is one multiply-add long. Everything float32; y in any storage type.
+template <class TOut>
+__global__ void lru_scan_kernel(const float* __restrict__ ug, const float* __restrict__ gates,
+                                const float* __restrict__ rb, const float* __restrict__ ib,
+                                const float* __restrict__ lam, float rate, float* __restrict__ state,
+                                const int* __restrict__ seq_starts, const int* __restrict__ slots,
+                                TOut* __restrict__ y, int W, int bw) {
+    const int seq = blockIdx.x;
+    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= W) return;
+    const int gc = (c / bw) * 2 * bw + c % bw;         // the channel's place among a row's gates
+    const int first = seq_starts[seq], last = seq_starts[seq + 1];
+    float* S_mem = state + (size_t)slots[seq] * W + c;
+    float S = *S_mem;
+    const float z = lam[c];
+    const float step = -rate * (z > 20.f ? z : log1pf(expf(z)));
+    const float rbc = rb[c], ibc = ib[c];
+#pragma unroll 4
+    for (int t = first; t < last; ++t) {
+        const float r = 1.0f / (1.0f + expf(-(gates[(size_t)t * 2 * W + gc] + rbc)));
+        const float i = 1.0f / (1.0f + expf(-(gates[(size_t)t * 2 * W + gc + bw] + ibc)));
+        const float log_a = step * r;
+        const float a = expf(log_a);
+        const float in = sqrtf(-expm1f(2.0f * log_a)) * i * ug[(size_t)t * 2 * W + c];
+        S = fmaf(a, S, in);
+        y[(size_t)t * W + c] = hb_from_float<TOut>(S * ug[(size_t)t * 2 * W + W + c]);
+    }
+    *S_mem = S;
+}
+
+extern "C" int hb_lru_scan(const float* ug, const float* gates, const float* rb, const float* ib, const float* lam,
+                           float rate, float* state, const int* seq_starts, const int* slots, void* y, int y_dtype,
+                           int B, int W, int bw, hipStream_t stream) {
+    HB_REQUIRE(B > 0 && W > 0 && B <= 65535, "recurrent unit: empty input or too many sequences for the grid");
+    HB_REQUIRE(bw > 0 && W % bw == 0, "recurrent unit: %d channels in blocks of %d", W, bw);
+    const int threads = W >= 4096 ? 256 : 64;          // (few channels: more, smaller workgroups over the CUs)
+    const dim3 grid(B, (W + threads - 1) / threads);
+    if (y_dtype == HB_F32)
+        lru_scan_kernel<float><<<grid, threads, 0, stream>>>(ug, gates, rb, ib, lam, rate, state, seq_starts, slots, (float*)y, W, bw);
+    else if (y_dtype == HB_BF16)
+        lru_scan_kernel<bf16><<<grid, threads, 0, stream>>>(ug, gates, rb, ib, lam, rate, state, seq_starts, slots, (bf16*)y, W, bw);
+    else
+        HB_REQUIRE(false, "recurrent unit: unknown output dtype %d", y_dtype);
+    HB_CHECK_LAUNCH("lru_scan");
     return 0;
 }
 
@@ -114,6 +232,9 @@ extern "C" int hb_conv_silu(const float* proj, int ld, const float* taps, float*
 // with 8 tokens a group the kernel took that latency over 8 a token. (8 where 16 would not fit 64 KB of LDS.)
 // CH: the decay is a factor a row of S (a key channel) instead of one a head: decay [T, heads x D] holds
 // the factors themselves (hb_channel_decay makes them), and they come through the ring beside k and q.
+// DELTA false (with CH): a linear attention with a decay a key channel, S <- diag(g) S + k v^T, o = S^T q: the same
+// walk without the correction along the key (u = v) and without beta.
+// C is what lies between two rows of qkv (at least the channels named above); o is multiplied by out_scale.
 #define DELTA_SUB_OF(DP, CH) ((CH) ? ((DP) >= 128 ? 8 : 16) : ((DP) >= 256 ? 8 : 16))
 #define DELTA_RING_OF(DP, CH) (((CH) && (DP) >= 256) ? 2 : 3)
 
@@ -138,13 +259,13 @@ __device__ __forceinline__ float delta_column_sum(float v) {
     return v;
 }
 
-template <int LPC, int DELTA_PER, bool CH>
+template <int LPC, int DELTA_PER, bool CH, bool DELTA>
 __global__ void __launch_bounds__(HB_WAVE)
 gated_delta_kernel(const float* __restrict__ qkv, int C, const float* __restrict__ proj, int ld, int b_off,
                    int a_off, const float* __restrict__ A_log, const float* __restrict__ dt_bias,
                    const float* __restrict__ decay, float* __restrict__ state,
                    const int* __restrict__ seq_starts, const int* __restrict__ slots,
-                   float* __restrict__ out, int kv_heads, int heads, int D, int V) {
+                   float* __restrict__ out, int kv_heads, int heads, int D, int V, float out_scale) {
     constexpr int COLS = HB_WAVE / LPC;
     constexpr int DP = LPC * DELTA_PER;                 // D rounded up to what the lanes hold
     constexpr int DELTA_RING = DELTA_RING_OF(DP, CH);
@@ -219,7 +340,7 @@ gated_delta_kernel(const float* __restrict__ qkv, int C, const float* __restrict
                 const float softplus = z > 20.f ? z : log1pf(expf(z));
                 g_reg = expf(rate * softplus);
             }
-            beta_reg = 1.0f / (1.0f + expf(-proj[(size_t)(t0 + lane) * ld + b_off + h]));
+            if (DELTA) beta_reg = 1.0f / (1.0f + expf(-proj[(size_t)(t0 + lane) * ld + b_off + h]));
         }
     };
     // ... and from the registers into the ring
@@ -270,10 +391,13 @@ gated_delta_kernel(const float* __restrict__ qkv, int C, const float* __restrict
                     const float4 gg = *(const float4*)&kq_ring[s0 + i][2 * DP + d0 + e];
                     S[e] *= gg.x, S[e + 1] *= gg.y, S[e + 2] *= gg.z, S[e + 3] *= gg.w;
                 }
+                float u = vc;
+                if (DELTA) {
 #pragma unroll
-                for (int e = 0; e < DELTA_PER; ++e) d4[e & 3] = fmaf(S[e], kc[e], d4[e & 3]);
-                const float dot = delta_column_sum<LPC>((d4[0] + d4[1]) + (d4[2] + d4[3]));
-                const float u = beta * (vc - dot);
+                    for (int e = 0; e < DELTA_PER; ++e) d4[e & 3] = fmaf(S[e], kc[e], d4[e & 3]);
+                    const float dot = delta_column_sum<LPC>((d4[0] + d4[1]) + (d4[2] + d4[3]));
+                    u = beta * (vc - dot);
+                }
                 float o4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int e = 0; e < DELTA_PER; ++e) {
@@ -281,7 +405,7 @@ gated_delta_kernel(const float* __restrict__ qkv, int C, const float* __restrict
                     o4[e & 3] = fmaf(S[e], qc[e], o4[e & 3]);
                 }
                 const float o = delta_column_sum<LPC>((o4[0] + o4[1]) + (o4[2] + o4[3]));
-                if (live && part == 0) out[(size_t)(t0 + i) * heads * V + h * V + col] = o;
+                if (live && part == 0) out[(size_t)(t0 + i) * heads * V + h * V + col] = o * out_scale;
                 continue;
             }
             // g (S^T k) = (g S)^T k: the dot product runs on the old numbers, in four partial sums, and the
@@ -298,7 +422,7 @@ gated_delta_kernel(const float* __restrict__ qkv, int C, const float* __restrict
                 o4[e & 3] = fmaf(S[e], qc[e], o4[e & 3]);
             }
             const float o = delta_column_sum<LPC>((o4[0] + o4[1]) + (o4[2] + o4[3]));
-            if (live && part == 0) out[(size_t)(t0 + i) * heads * V + h * V + col] = o;
+            if (live && part == 0) out[(size_t)(t0 + i) * heads * V + h * V + col] = o * out_scale;
         }
         if (ahead) stash(p + DELTA_RING - 1);           // (the place of the group before this one)
         __syncthreads();
@@ -312,14 +436,16 @@ gated_delta_kernel(const float* __restrict__ qkv, int C, const float* __restrict
 
 // decay null: one factor a head, from the projection's column a_off + h, A_log and dt_bias.
 // decay [T, heads x D]: a factor a key channel, as given (a_off, A_log and dt_bias are not read).
+// correction 0 (a decay a key channel must be given): the linear attention, S <- diag(g) S + k v^T; proj is not read.
 extern "C" int hb_gated_delta(const float* qkv, int C, const float* proj, int ld, int b_off, int a_off,
                               const float* A_log, const float* dt_bias, const float* decay, float* state,
                               const int* seq_starts,
                               const int* slots, float* out, int B, int kv_heads, int heads, int D, int V,
-                              hipStream_t stream) {
+                              int correction, float out_scale, hipStream_t stream) {
+    HB_REQUIRE(correction || decay, "linear attention: the walk without a correction takes a decay a key channel");
     HB_REQUIRE(B > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "delta rule: %d heads on %d key heads", heads, kv_heads);
     HB_REQUIRE(D > 0 && D <= 256, "delta rule: keys of %d, the kernel takes 1 to 256", D);
-    HB_REQUIRE(V > 0 && C == 2 * kv_heads * D + heads * V, "delta rule: %d channels do not fit the heads", C);
+    HB_REQUIRE(V > 0 && C >= 2 * kv_heads * D + heads * V, "delta rule: rows of %d do not hold the heads' channels", C);
     HB_REQUIRE(B <= 65535 && heads <= 65535, "delta rule: too many sequences or heads for the grid");
     // Lanes a column x numbers a lane. Few waves (one prompt of a model of up to 16 heads of 128 columns): 8 numbers a lane, so that a token's step is
     // short (the chain is what counts: 2,048 tokens of 16 heads of 128 x 128 take 0.97 ms with 16 numbers a
@@ -333,12 +459,15 @@ extern "C" int hb_gated_delta(const float* qkv, int C, const float* proj, int ld
     const dim3 grid(B, heads, (V + cols - 1) / cols);
 #define HB_DELTA(L, P)                                                                                            \
     do {                                                                                                          \
-        if (decay)                                                                                                \
-            gated_delta_kernel<L, P, true><<<grid, HB_WAVE, 0, stream>>>(qkv, C, proj, ld, b_off, a_off, A_log,   \
-                dt_bias, decay, state, seq_starts, slots, out, kv_heads, heads, D, V);                            \
+        if (decay && !correction)                                                                                 \
+            gated_delta_kernel<L, P, true, false><<<grid, HB_WAVE, 0, stream>>>(qkv, C, proj, ld, b_off, a_off, A_log, \
+                dt_bias, decay, state, seq_starts, slots, out, kv_heads, heads, D, V, out_scale);                 \
+        else if (decay)                                                                                           \
+            gated_delta_kernel<L, P, true, true><<<grid, HB_WAVE, 0, stream>>>(qkv, C, proj, ld, b_off, a_off, A_log, \
+                dt_bias, decay, state, seq_starts, slots, out, kv_heads, heads, D, V, out_scale);                 \
         else                                                                                                      \
-            gated_delta_kernel<L, P, false><<<grid, HB_WAVE, 0, stream>>>(qkv, C, proj, ld, b_off, a_off, A_log,  \
-                dt_bias, decay, state, seq_starts, slots, out, kv_heads, heads, D, V);                            \
+            gated_delta_kernel<L, P, false, true><<<grid, HB_WAVE, 0, stream>>>(qkv, C, proj, ld, b_off, a_off, A_log, \
+                dt_bias, decay, state, seq_starts, slots, out, kv_heads, heads, D, V, out_scale);                 \
     } while (0)
     if (wide) {
         if (lpc == 1) HB_DELTA(1, 8);

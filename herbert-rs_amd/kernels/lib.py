@@ -24,7 +24,12 @@ SIGNATURES = {
         "hb_rmsnorm": [_P, _P, _P, _I, _P, _I, _I, _F, _P],
         "hb_qk_norm_rope_write": [_P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I,
                                   _I, _I, _I, _I, _F, _I, _I, ctypes.c_size_t, _F, _I, _P],
-        "hb_swiglu": [_P, _P, _I, _I, _I, _P],
+        "hb_swiglu": [_P, _P, _I, _I, _I, _I, _P],
+        "hb_rmsnorm_scaled_sum": [_P, _P, _P, _P, _P, _I, _I, _I, _F, _P],
+        "hb_normed_pair": [_P, _P, _F, _P, _P, _F, _P, _I, _I, _F, _I, _P],
+        "hb_filter_norm_rotate_write": [_P, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P,
+                                        _I, _I, _I, _I, _I, _I, _I, _F, _P],
+        "hb_gate_heads": [_P, _I, _P, _I, _I, _P, _I, _I, _I, _I, _P],
         "hb_fill_u32": [_P, _U32, _SZ, _P],
         "hb_layernorm": [_P, _P, _F, _P, _P, _I, _P, _I, _I, _F, _P],
         "hb_scale": [_P, _F, _SZ, _P],
@@ -33,12 +38,15 @@ SIGNATURES = {
     },
     "gemm_plain": {
         "hb_gemm_plain": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
-        "hb_gemm_plain_short_k": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P],
+        "hb_gemm_plain_short_k": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _I, _F, _P],
         "hb_gemm_plain_batched": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _SZ, _SZ, _SZ, _P],
     },
     "recurrent": {
         "hb_conv_silu": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _I, _P],
-        "hb_gated_delta": [_P, _I, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+        "hb_gated_delta": [_P, _I, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
+        "hb_filter_state": [_P, _I, _P, _P, _P, _I, _I, _I, _P, _P],
+        "hb_lru_inputs": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+        "hb_lru_scan": [_P, _P, _P, _P, _P, _F, _P, _P, _P, _P, _I, _I, _I, _I, _P],
         "hb_gated_head_norm": [_P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _P],
         "hb_channel_decay": [_P, _I, _P, _P, _P, _I, _I, _I, _P],
     },
@@ -55,7 +63,7 @@ SIGNATURES = {
         "hb_grouped_mfma": [_P, _I, _SZ, _P, _I, _I, _P, _I, _SZ, _I, _P, _I, _P, _P, _P, _I, _I, _I, _F, _F, _F, _I, _P],
     },
     "attention_plain": {
-        "hb_attention_plain": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+        "hb_attention_plain": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P],
     },
     "sampling": {
         "hb_argmax": [_P, _I, _I, _I, _P, _P, _P, _I, _P],

@@ -187,9 +187,12 @@ def qk_norm_rope_write(qkv, q_norm_w, k_norm_w, cos, sin, rot_dims, meta, cache,
              n_slices, stride, coef, every, _stream())
 
 
-def attention_plain(q, meta, cache, out, nq, nkv, hd, scale, window):
-    """Causal (and windowed) attention of every token over its slot's pages."""
+def attention_plain(q, meta, cache, out, nq, nkv, hd, scale, window, sinks=None):
+    """Causal (and windowed) attention of every token over its slot's pages. sinks f32 [nq]: the softmax's
+    denominator of head h also holds exp(sinks[h])."""
     T = q.shape[0]
+    if sinks is not None:
+        _check(sinks, "sinks", torch.float32, (nq,))
     _check(q, "q", cache.k.dtype, (T, nq * hd))
     _check(out, "out", cache.k.dtype, (T, nq * hd))
     _check_paged(meta, cache, T)
@@ -199,18 +202,23 @@ def attention_plain(q, meta, cache, out, nq, nkv, hd, scale, window):
              cache.v.data_ptr(), out.data_ptr(), dtype_code(q), meta.positions.data_ptr(),
              meta.seq_of.data_ptr(), meta.slots.data_ptr(), cache.page_table.data_ptr(),
              cache.page_table.shape[1], cache.page_size, T, nq, nkv, hd, float(scale),
-             int(window or 0), _stream())
+             int(window or 0), _ptr(sinks), _stream())
 
 
-def swiglu(gu, out):
-    """out[t, i] = silu(gu[t, i]) * gu[t, I + i]; gu f32 [T, 2I]."""
+GLU_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def swiglu(gu, out, activation="silu"):
+    """out[t, i] = f(gu[t, i]) * gu[t, I + i]; gu f32 [T, 2I]; f "silu" or "gelu_tanh"."""
+    if activation not in GLU_ACTIVATIONS:
+        raise BackendError(f"gated linear unit: unknown activation {activation!r}")
     _check(gu, "gate_up", torch.float32, (None, None))
     T, two_i = gu.shape
     if two_i % 2:
         raise BackendError("swiglu: the input's width must be even")
     _check(out, "out", None, (T, two_i // 2))
     lib.call("elementwise", "hb_swiglu", gu.data_ptr(), out.data_ptr(), dtype_code(out), T, two_i // 2,
-             _stream())
+             GLU_ACTIVATIONS[activation], _stream())
 
 
 def fill_u32(t, value):
@@ -452,7 +460,8 @@ def gemm_plain_columns(a, col0, K, w, c, accumulate=False, decay=None):
     more and smaller workgroups than the tiled one, which a short k leaves with few.)
     decay (a_log f32 [N / D], dt_bias f32 [N], D): the sums are a decay's pre-activations, and c (float32, not
     added to) takes the decays themselves, exp(-exp(a_log[n // D]) softplus(sum + dt_bias[n])), as
-    `recurrent.channel_decay` makes them from rows in memory."""
+    `recurrent.channel_decay` makes them from rows in memory.
+    decay ("sigmoid_root", bias f32 [N], root): c takes sigmoid(sum + bias[n])^root instead."""
     _check(a, "a", None, (None, None))
     _check(w, "w", None, (None, K))
     M, lda = a.shape
@@ -463,7 +472,15 @@ def gemm_plain_columns(a, col0, K, w, c, accumulate=False, decay=None):
     if accumulate and c.dtype != torch.float32:
         raise BackendError("gemm: accumulation needs a float32 output")
     a_log = dt_bias = D = 0
-    if decay is not None:
+    root = 0.0
+    if decay is not None and decay[0] == "sigmoid_root":
+        _, bias, root = decay
+        if accumulate or c.dtype != torch.float32:
+            raise BackendError("gemm: a decay is float32, stored and not added to")
+        _check(bias, "decay bias", torch.float32, (N,))
+        a_log = dt_bias = bias.data_ptr()
+        D = 1
+    elif decay is not None:
         rate, bias, D = decay
         if accumulate or c.dtype != torch.float32 or D <= 0 or N % D:
             raise BackendError("gemm: a decay is float32, stored and not added to, its columns whole heads")
@@ -472,4 +489,85 @@ def gemm_plain_columns(a, col0, K, w, c, accumulate=False, decay=None):
         a_log, dt_bias = rate.data_ptr(), bias.data_ptr()
     lib.call("gemm_plain", "hb_gemm_plain_short_k", a.data_ptr() + col0 * a.element_size(), dtype_code(a), w.data_ptr(),
              dtype_code(w), c.data_ptr(), dtype_code(c), M, N, K, lda, K, N, 1 if accumulate else 0, a_log, dt_bias,
-             int(D), _stream())
+             int(D), float(root), _stream())
+
+
+def rmsnorm_scaled_sum(x, delta, factors, weight, out, eps):
+    """x += factors * delta (a factor a column), in place, then out = x / rms(x) * weight; x, delta f32 [T, H],
+    factors f32 [H]. out None (weight may then be None): only the sum."""
+    _check(x, "x", torch.float32, (None, None))
+    T, H = x.shape
+    _check(delta, "delta", torch.float32, (T, H))
+    _check(factors, "factors", torch.float32, (H,))
+    if out is not None:
+        _check(weight, "weight", torch.float32, (H,))
+        _check(out, "out", None, (T, H))
+        if out.data_ptr() in (x.data_ptr(), delta.data_ptr()):
+            raise BackendError("rmsnorm: the normed rows must be other rows than the sum's")
+    lib.call("elementwise", "hb_rmsnorm_scaled_sum", x.data_ptr(), delta.data_ptr(), factors.data_ptr(), _ptr(weight),
+             _ptr(out), dtype_code(out) if out is not None else F32, T, H, float(eps), _stream())
+
+
+def normed_pair(a, wa, ca, b, wb, cb, out, eps, accumulate=False):
+    """out (+)= ca * a / rms(a) * wa + cb * b / rms(b) * wb, row by row; all f32 [T, H], weights [H]."""
+    _check(a, "a", torch.float32, (None, None))
+    T, H = a.shape
+    _check(b, "b", torch.float32, (T, H))
+    _check(out, "out", torch.float32, (T, H))
+    _check(wa, "wa", torch.float32, (H,))
+    _check(wb, "wb", torch.float32, (H,))
+    lib.call("elementwise", "hb_normed_pair", a.data_ptr(), wa.data_ptr(), float(ca), b.data_ptr(), wb.data_ptr(), float(cb),
+             out.data_ptr(), T, H, float(eps), 1 if accumulate else 0, _stream())
+
+
+def filter_norm_rotate_write(proj, taps, filter_state, q_norm_w, k_norm_w, rates, rot_dims, meta, cache, q_out,
+                             nq, nkv, dim, vdim, hd, eps):
+    """The first columns of proj's rows (f32 [T, ld]) are [nq x dim queries | nkv x dim keys | nkv x vdim values]:
+    filtered along time (taps f32 [C, K] with the slot's last inputs in filter_state f32 [slots, K - 1, C]; None:
+    no filter), queries and keys each normed over the whole projection (weights [nq x dim], [nkv x dim]; None:
+    no norm), neighbouring pairs of the first rot_dims entries of every head turned by position x rates (f64
+    [rot_dims / 2]; None: no rotation); q to q_out [T, nq x hd], keys and values to the token's page, heads kept
+    at hd with zeros beyond their own size. The filter's state is moved on by recurrent.filter_state."""
+    T, ld = proj.shape
+    C = (nq + nkv) * dim + nkv * vdim
+    _check(proj, "proj", torch.float32, (T, ld))
+    K = 0
+    if taps is not None:
+        K = taps.shape[1]
+        _check(taps, "taps", torch.float32, (C, K))
+        if K > 1:
+            _check(filter_state, "filter_state", torch.float32, (None, K - 1, C))
+    if q_norm_w is not None:
+        _check(q_norm_w, "q_norm", torch.float32, (nq * dim,))
+    if k_norm_w is not None:
+        _check(k_norm_w, "k_norm", torch.float32, (nkv * dim,))
+    if rates is not None:
+        _check(rates, "rates", torch.float64, (rot_dims // 2,))
+    _check_paged(meta, cache, T)
+    _check(meta.seq_starts, "seq_starts", torch.int32, (meta.num_seqs + 1,))
+    _check(q_out, "q_out", cache.k.dtype, (T, nq * hd))
+    if tuple(cache.k.shape[1:]) != (nkv, cache.page_size, hd):
+        raise BackendError(f"cache pages {list(cache.k.shape)} do not fit {nkv} kv heads of {hd}")
+    if ld < C or hd < max(dim, vdim):
+        raise BackendError(f"filtered attention: rows of {ld} for {C} channels, heads of {dim} and {vdim} kept at {hd}")
+    lib.call("elementwise", "hb_filter_norm_rotate_write", proj.data_ptr(), ld, _ptr(taps), K,
+             _ptr(filter_state) if K > 1 else None, _ptr(q_norm_w), _ptr(k_norm_w), _ptr(rates), int(rot_dims),
+             meta.positions.data_ptr(), meta.seq_of.data_ptr(), meta.seq_starts.data_ptr(), meta.slots.data_ptr(),
+             cache.page_table.data_ptr(), cache.page_table.shape[1], cache.page_size, q_out.data_ptr(),
+             cache.k.data_ptr(), cache.v.data_ptr(), dtype_code(q_out), T, nq, nkv, dim, vdim, hd, float(eps), _stream())
+
+
+def gate_heads(attn, gate_rows, g_off, out, nq, hd, vdim):
+    """out[t, h vdim + d] = attn[t, h hd + d] * sigmoid(gate_rows[t, g_off + h vdim + d]), d < vdim; attn [T, nq hd]
+    and out [T, nq vdim] of one dtype, gate_rows f32 [T, ld] (None: no gate, the heads only leave at their own size)."""
+    T = attn.shape[0]
+    _check(attn, "attn", None, (T, nq * hd))
+    _check(out, "out", attn.dtype, (T, nq * vdim))
+    ld = 0
+    if gate_rows is not None:
+        _check(gate_rows, "gate", torch.float32, (T, None))
+        ld = gate_rows.shape[1]
+        if g_off < 0 or g_off + nq * vdim > ld:
+            raise BackendError("gate: its columns lie outside the rows")
+    lib.call("elementwise", "hb_gate_heads", attn.data_ptr(), dtype_code(attn), _ptr(gate_rows), ld, int(g_off),
+             out.data_ptr(), T, nq, hd, vdim, _stream())

@@ -34,13 +34,31 @@ def conv_silu(proj, taps, conv_state, meta, out, n_unit, unit_dim, n_scaled, sca
              _stream())
 
 
-def gated_delta(qkv, proj, b_off, a_off, a_log, dt_bias, state, meta, out, kv_heads, heads, D, V, decay=None):
-    """The delta rule over every sequence of the step; qkv f32 [T, 2 kv_heads D + heads V] (queries,
-    keys, values), proj f32 [T, ld] with column b_off + h (beta's pre-activation) and a_off + h (the
+def gated_delta(qkv, proj, b_off, a_off, a_log, dt_bias, state, meta, out, kv_heads, heads, D, V, decay=None,
+                correction=True, out_scale=1.0):
+    """The delta rule over every sequence of the step; qkv f32 [T, at least 2 kv_heads D + heads V] (queries,
+    keys, values in a row's first columns), proj f32 [T, ld] with column b_off + h (beta's pre-activation) and a_off + h (the
     decay's), state f32 [slots, heads, D, V] advanced in place, out f32 [T, heads V].
     decay f32 [T, heads D]: a factor a key channel, as `channel_decay` leaves it; a_off, a_log and
-    dt_bias are then not read (they may be None)."""
+    dt_bias are then not read (they may be None). correction False (a decay a key channel must be given):
+    the linear attention S <- diag(decay) S + k v^T, o = S^T q; proj is then not read (it may be None).
+    out_scale: o is multiplied by it."""
     T, C = qkv.shape
+    if not correction:
+        if decay is None:
+            raise BackendError("linear attention: the walk without a correction takes a decay a key channel")
+        _check(decay, "decay", torch.float32, (T, heads * D))
+        _check(qkv, "qkv", torch.float32, (T, None))
+        _check(state, "state", torch.float32, (None, heads, D, V))
+        _check(out, "out", torch.float32, (T, heads * V))
+        _check(meta.seq_starts, "seq_starts", torch.int32, (meta.num_seqs + 1,))
+        _check(meta.slots, "slots", torch.int32, (meta.num_seqs,))
+        if heads % kv_heads or not 0 < D <= MAX_KEY_DIM or C < 2 * kv_heads * D + heads * V:
+            raise BackendError(f"linear attention: {heads} heads on {kv_heads} key heads of {D} in rows of {C}")
+        lib.call("recurrent", "hb_gated_delta", qkv.data_ptr(), C, None, 0, 0, 0, None, None, decay.data_ptr(),
+                 state.data_ptr(), meta.seq_starts.data_ptr(), meta.slots.data_ptr(), out.data_ptr(), meta.num_seqs,
+                 kv_heads, heads, D, V, 0, float(out_scale), _stream())
+        return
     if decay is not None:
         _check(decay, "decay", torch.float32, (T, heads * D))
         a_off = 0
@@ -62,7 +80,7 @@ def gated_delta(qkv, proj, b_off, a_off, a_log, dt_bias, state, meta, out, kv_he
              None if decay is not None else a_log.data_ptr(), None if decay is not None else dt_bias.data_ptr(),
              None if decay is None else decay.data_ptr(), state.data_ptr(), meta.seq_starts.data_ptr(),
              meta.slots.data_ptr(),
-             out.data_ptr(), meta.num_seqs, kv_heads, heads, D, V, _stream())
+             out.data_ptr(), meta.num_seqs, kv_heads, heads, D, V, 1, float(out_scale), _stream())
 
 
 def gated_head_norm(o, proj, g_off, weight, out, heads, V, eps, gate="silu"):
@@ -94,3 +112,66 @@ def channel_decay(z, z_off, a_log, dt_bias, out, heads, D):
         raise BackendError("channel decay: the pre-activations lie outside their rows")
     lib.call("recurrent", "hb_channel_decay", z.data_ptr() + 4 * z_off, ld, a_log.data_ptr(), dt_bias.data_ptr(),
              out.data_ptr(), T, heads, D, _stream())
+
+
+def filter_state(proj, conv_state, meta, C, K, bias=None):
+    """After a step: conv_state (f32 [slots, K - 1, C]) takes the last K - 1 inputs of each sequence, the first C
+    columns of proj's rows (f32 [T, ld]) plus bias (f32 [C]) if given. For mixers that filter in a kernel of
+    their own."""
+    T, ld = proj.shape
+    _check(proj, "proj", torch.float32, (T, ld))
+    if K <= 1:
+        return
+    _check(conv_state, "conv_state", torch.float32, (None, K - 1, C))
+    _check(meta.seq_starts, "seq_starts", torch.int32, (meta.num_seqs + 1,))
+    _check(meta.slots, "slots", torch.int32, (meta.num_seqs,))
+    if bias is not None:
+        _check(bias, "bias", torch.float32, (C,))
+    if ld < C or K > MAX_TAPS:
+        raise BackendError(f"filter state: {C} channels of {K} taps in rows of {ld}")
+    lib.call("recurrent", "hb_filter_state", proj.data_ptr(), ld, conv_state.data_ptr(), meta.seq_starts.data_ptr(),
+             meta.slots.data_ptr(), meta.num_seqs, C, K, None if bias is None else bias.data_ptr(), _stream())
+
+
+def lru_inputs(proj, bx, by, taps, filter_bias, conv_state, meta, out):
+    """The two branches of a gated linear recurrent unit from the projection's rows [x | y] (f32 [T, ld], W
+    channels each): out f32 [T, 2 W] = [filter(x + bx) + filter_bias | gelu_tanh(y + by)]; taps f32 [W, K],
+    conv_state f32 [slots, K - 1, W] (the inputs with their bias), moved on afterwards."""
+    T, ld = proj.shape
+    W, K = taps.shape
+    _check(proj, "proj", torch.float32, (T, ld))
+    _check(taps, "taps", torch.float32, (W, K))
+    for t, name in ((bx, "x bias"), (by, "y bias")):
+        _check(t, name, torch.float32, (W,))
+    if filter_bias is not None:
+        _check(filter_bias, "filter bias", torch.float32, (W,))
+    _check(conv_state, "conv_state", torch.float32, (None, max(K - 1, 1), W))
+    _check(out, "out", torch.float32, (T, 2 * W))
+    _check(meta.seq_of, "seq_of", torch.int32, (T,))
+    _check(meta.seq_starts, "seq_starts", torch.int32, (meta.num_seqs + 1,))
+    _check(meta.slots, "slots", torch.int32, (meta.num_seqs,))
+    if ld < 2 * W or not 1 <= K <= MAX_TAPS:
+        raise BackendError(f"recurrent unit: rows of {ld} for 2 x {W} channels, {K} taps")
+    lib.call("recurrent", "hb_lru_inputs", proj.data_ptr(), ld, bx.data_ptr(), by.data_ptr(), taps.data_ptr(),
+             None if filter_bias is None else filter_bias.data_ptr(), conv_state.data_ptr(), meta.seq_of.data_ptr(),
+             meta.seq_starts.data_ptr(), meta.slots.data_ptr(), out.data_ptr(), T, meta.num_seqs, W, K, _stream())
+
+
+def lru_scan(ug, gates, r_bias, i_bias, lam, rate, state, meta, out, block):
+    """The recurrence of every sequence of the step, channel by channel: with r = sigmoid(r_pre + r_bias),
+    i = sigmoid(i_pre + i_bias), a = exp(-rate r softplus(lam)): S <- a S + sqrt(1 - a^2) i u, out = S g, where
+    ug f32 [T, 2 W] = [u | g] and gates f32 [T, 2 W] holds, for every block of `block` channels, that block's
+    r_pre then its i_pre; state f32 [slots, W] advanced in place; out [T, W] in any dtype."""
+    T, W2 = ug.shape
+    W = W2 // 2
+    _check(ug, "ug", torch.float32, (T, 2 * W))
+    _check(gates, "gates", torch.float32, (T, 2 * W))
+    for t, name in ((r_bias, "r bias"), (i_bias, "i bias"), (lam, "lam")):
+        _check(t, name, torch.float32, (W,))
+    _check(state, "state", torch.float32, (None, W))
+    _check(out, "out", None, (T, W))
+    _check(meta.seq_starts, "seq_starts", torch.int32, (meta.num_seqs + 1,))
+    _check(meta.slots, "slots", torch.int32, (meta.num_seqs,))
+    lib.call("recurrent", "hb_lru_scan", ug.data_ptr(), gates.data_ptr(), r_bias.data_ptr(), i_bias.data_ptr(),
+             lam.data_ptr(), float(rate), state.data_ptr(), meta.seq_starts.data_ptr(), meta.slots.data_ptr(),
+             out.data_ptr(), dtype_code(out), meta.num_seqs, W, int(block), _stream())

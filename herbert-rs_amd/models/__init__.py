@@ -1,4 +1,4 @@
 """Architectures: each module turns its typed configuration into a ModelSpec and registers itself."""
-from . import modasun, qwen3, vipalorn
+from . import mefatar, modasun, qwen3, vipalorn
 
-__all__ = ["modasun", "qwen3", "vipalorn"]
+__all__ = ["mefatar", "modasun", "qwen3", "vipalorn"]

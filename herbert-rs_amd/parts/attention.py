@@ -15,6 +15,15 @@ reference does not have. Nor are these: values of another size than the keys
 that grows with the logarithm of its position (`q_temp=(coef, every)`: times
 1 + coef ln(floor((p + 1) / every) + 1) at position p, after norm and rotation).
 
+A further form of the part (not in the reference either), taken where any of these is asked for: `conv` (queries,
+keys and values pass a filter along time, channel by channel, directly after their projections; the last
+conv - 1 projected rows of a sequence are state beside its keys and values), `qk_norm="whole"` (queries, and keys,
+are normed over the whole projection at once, before they are split into heads, with a weight of that size),
+a position of the kind "rope_pairs" (neighbouring pairs turn), `sink` (the softmax's denominator of a head also
+holds exp(s_h), a stored number a head without key or value), `gate` (the joined heads times sigmoid(W_g y)
+before the output projection). Such a part filters, norms, rotates and writes the cache in one kernel of its
+own; rotation and values of another size than the keys go together there.
+
 The kernels keep one head size for queries, keys and values. Where a model's
 key and value sizes differ, or where the matrix cores (heads of 32, 64, 128)
 would otherwise refuse a head, the part runs them at a larger size whose
@@ -27,12 +36,22 @@ import math
 
 import torch
 
-from ..cache import KVNeed
-from ..kernels import mfma, ops
+from ..cache import KVNeed, StateNeed
+from ..kernels import mfma, ops, recurrent
 from ..weights import TensorNeed
 from .base import Part
 from .linear import Linear
 from .registry import register
+
+
+def _taps_init(shape, gen, device, std, norm_std):
+    """Taps near an average of the window, so that a random model's filter passes its input on."""
+    return 1.0 / shape[1] + 0.3 * torch.randn(shape, generator=gen, device=device, dtype=torch.float32)
+
+
+def _sink_init(shape, gen, device, std, norm_std):
+    """Sinks of a random model: around zero, so that they take a visible share of a short row's weight."""
+    return torch.randn(shape, generator=gen, device=device, dtype=torch.float32)
 
 
 @register("mixer", "attention")
@@ -41,15 +60,18 @@ class Attention(Part):
 
     def __init__(self, hidden_size, num_heads, num_kv_heads, head_dim, eps, position, names,
                  qk_norm=True, window=None, scale=None, shared=None, reads_cache_only=False,
-                 value_dim=None, q_temp=None):
-        """names: dict with q, k, v, o (and q_norm, k_norm when qk_norm is True) -> tensor names.
-        qk_norm: True (a weight [head_dim] each for queries and keys), "plain" (no weights) or False.
+                 value_dim=None, q_temp=None, conv=None, sink=False, gate=False):
+        """names: dict with q, k, v, o (and q_norm, k_norm when qk_norm is True or "whole"; q_conv, k_conv, v_conv
+        with conv; sink with sink; g with gate) -> tensor names.
+        qk_norm: True (a weight [head_dim] each for queries and keys), "plain" (no weights), "whole" (over all
+        heads of a token at once, weights of that size) or False.
+        conv: taps of a filter along time on queries, keys and values (None: none).
         reads_cache_only: the part has no k / v projections and attends over a cache that
         another entry of the schedule fills."""
         if num_heads % num_kv_heads:
             raise ValueError("num_heads must be divisible by num_kv_heads")
-        if qk_norm not in (True, False, "plain"):
-            raise ValueError(f"qk_norm is True, False or 'plain', not {qk_norm!r}")
+        if qk_norm not in (True, False, "plain", "whole"):
+            raise ValueError(f"qk_norm is True, False, 'plain' or 'whole', not {qk_norm!r}")
         self.hidden_size = int(hidden_size)
         self.nq = int(num_heads)
         self.nkv = int(num_kv_heads)
@@ -67,6 +89,21 @@ class Attention(Part):
         self.reads_cache_only = bool(reads_cache_only)
         self.position = shared.position(position)
         self.qkv = self.o = self.q_norm_w = self.k_norm_w = None
+        self.taps = int(conv) if conv else 0
+        self.sink, self.gate = bool(sink), bool(gate)
+        self.sink_w = self.taps_w = None
+        # the form with a kernel of its own before the attention (see the module's text)
+        self.prepared = bool(self.taps or self.sink or self.gate or qk_norm == "whole"
+                             or hasattr(self.position, "pair_rates"))
+        if self.prepared:
+            if self.reads_cache_only or self.q_temp is not None or qk_norm in (True, "plain") or \
+                    self.position.rotation() is not None:
+                raise ValueError("a filter, a norm over the whole projection, a rotation of pairs, a sink or a gate "
+                                 "go with a cache of the part's own, no per-head norm, no growing query and no "
+                                 "rotation of halves")
+            if self.taps > recurrent.MAX_TAPS:
+                raise ValueError(f"the filter takes up to {recurrent.MAX_TAPS} taps, not {self.taps}")
+            self.stores_fresh_rows = True        # its output projection stores into rows that hold nothing yet
 
     @property
     def q_dim(self):
@@ -85,10 +122,25 @@ class Attention(Part):
     def kernel_scale(self):
         return self.scale * self.dim / self.hd if self.qk_norm else self.scale
 
+    @property
+    def channels(self):
+        """Channels that pass the filter: queries, keys, values."""
+        return (self.nq + self.nkv) * self.dim + self.nkv * self.vdim
+
     def tensor_needs(self):
         n, W = self.names, self.hidden_size
         needs = {n["q"]: TensorNeed((self.nq * self.dim, W)),
                  n["o"]: TensorNeed((W, self.nq * self.vdim))}
+        if self.qk_norm == "whole":
+            needs[n["q_norm"]] = TensorNeed((self.nq * self.dim,), "scale")
+            needs[n["k_norm"]] = TensorNeed((self.nkv * self.dim,), "scale")
+        if self.taps:
+            for key, rows in (("q_conv", self.nq * self.dim), ("k_conv", self.nkv * self.dim), ("v_conv", self.nkv * self.vdim)):
+                needs[n[key]] = TensorNeed((rows, self.taps), "taps", _taps_init)
+        if self.sink:
+            needs[n["sink"]] = TensorNeed((self.nq,), "bias", _sink_init)
+        if self.gate:
+            needs[n["g"]] = TensorNeed((self.nq * self.vdim, W))
         if not self.reads_cache_only:
             needs[n["k"]] = TensorNeed((self.nkv * self.dim, W))
             needs[n["v"]] = TensorNeed((self.nkv * self.vdim, W))
@@ -102,6 +154,12 @@ class Attention(Part):
         """The head size the kernels run at: the larger of keys and values, and in bfloat16 the next size
         that the matrix cores take, unless the rotation or a cache that another entry fills forbids it."""
         size = max(self.dim, self.vdim)
+        if self.prepared:
+            if rt.dtype == torch.bfloat16:
+                for takes in mfma.ATTENTION_HEAD_DIMS:
+                    if size <= takes:
+                        return takes
+            return size
         if self.position.rotation() is not None or self.reads_cache_only:
             if self.vdim != self.dim:
                 raise ValueError("values of another size than the keys go with no rotation and a cache of the part's own")
@@ -129,9 +187,52 @@ class Attention(Part):
     def cache_need(self):
         if self.reads_cache_only:
             return None
+        if self.taps > 1:
+            return (KVNeed(self.nkv, self.hd, self.window), StateNeed((self.taps - 1, self.channels), torch.float32))
         return KVNeed(self.nkv, self.hd, self.window)
 
+    def _load_prepared(self, tensors, rt):
+        n = self.names
+        self.hd = self._kept_size(rt)
+        # one fused projection [q | k | v | gate], the heads at their own sizes: the kernel that follows reads
+        # its float32 sums where they lie and keeps the heads at the size the attention runs at
+        rows = [tensors[n[k]].to(rt.device) for k in ("q", "k", "v") + (("g",) if self.gate else ())]
+        self.qkv = Linear(rt.weight(torch.cat(rows, 0)), scratch=rt.scratch)
+        self.proj_width = self.channels + (self.nq * self.vdim if self.gate else 0)
+        self.o = Linear(rt.weight(tensors[n["o"]]), scratch=rt.scratch)
+        if self.qk_norm == "whole":
+            self.q_norm_w = rt.weight(tensors[n["q_norm"]], matrix=False)
+            self.k_norm_w = rt.weight(tensors[n["k_norm"]], matrix=False)
+        if self.taps:
+            self.taps_w = torch.cat([rt.weight(tensors[n[k]], matrix=False) for k in ("q_conv", "k_conv", "v_conv")],
+                                    0).contiguous()
+        if self.sink:
+            self.sink_w = rt.weight(tensors[n["sink"]], matrix=False)
+
+    def _forward_prepared(self, ctx, y, x):
+        rt = ctx.rt
+        T = x.shape[0]
+        kv = ctx.cache.kv_view(ctx.cache_entry)
+        proj = rt.buffer("attn_proj", (T, self.proj_width), torch.float32)
+        self.qkv.forward(y, proj)
+        q = rt.buffer("q", (T, self.q_dim))
+        state = ctx.cache.state_views(ctx.cache_entry)[0] if self.taps > 1 else None
+        rates, rot_dims = self.position.pair_rates() if hasattr(self.position, "pair_rates") else (None, 0)
+        ops.filter_norm_rotate_write(proj, self.taps_w, state, self.q_norm_w, self.k_norm_w, rates, rot_dims, ctx.meta,
+                                     kv, q, self.nq, self.nkv, self.dim, self.vdim, self.hd, self.eps)
+        if self.taps > 1:
+            recurrent.filter_state(proj, state, ctx.meta, self.channels, self.taps)
+        attn = rt.buffer("attn", (T, self.q_dim))
+        self.attend(ctx, q, kv, attn)
+        # the heads leave at their own size, each entry times its gate
+        gated = rt.buffer("attn_gated", (T, self.nq * self.vdim))
+        ops.gate_heads(attn, proj if self.gate else None, self.channels, gated, self.nq, self.hd, self.vdim)
+        self.o.forward(gated, x, accumulate=ctx.adds_to(x))
+
     def load(self, tensors, rt):
+        if self.prepared:
+            self._load_prepared(tensors, rt)
+            return
         n = self.names
         self.hd = kept = self._kept_size(rt)
         rows = [self._heads_padded(tensors[n["q"]].to(rt.device), self.nq, self.dim, kept)]
@@ -153,6 +254,8 @@ class Attention(Part):
     def forward_from_residual(self, ctx, x, norm):
         """With few rows and bfloat16 weights no norm kernel runs: the projection takes what the
         product before left of the norm, or else does the norm itself on the way."""
+        if self.prepared:
+            return False
         handed = ctx.take_handed(self.qkv, x)
         if handed is not None:
             self.forward(ctx, handed.xg, x, row_scale=handed.row_scale())
@@ -168,6 +271,9 @@ class Attention(Part):
         self.o.forward(attn, x, accumulate=True, leave=None if left is None else left.leave())
 
     def forward(self, ctx, y, x, fused_norm=None, row_scale=None):
+        if self.prepared:
+            self._forward_prepared(ctx, y, x)
+            return
         rt = ctx.rt
         T = x.shape[0]
         kv = ctx.cache.kv_view(ctx.cache_entry)
@@ -215,9 +321,13 @@ class Attention(Part):
         self.project_out(ctx, attn, x)
 
     def attend(self, ctx, q, kv, out):
+        scale = self.scale if self.prepared else self.kernel_scale
+        if self.sink_w is not None:
+            ops.attention_plain(q, ctx.meta, kv, out, self.nq, self.nkv, self.hd, scale, self.window, sinks=self.sink_w)
+            return
         if q.dtype == torch.bfloat16:
             if mfma.attention_supported(q, kv, self.nq, self.nkv, self.hd):
-                mfma.attention(q, ctx.meta, kv, out, self.nq, self.nkv, self.hd, self.kernel_scale, self.window,
+                mfma.attention(q, ctx.meta, kv, out, self.nq, self.nkv, self.hd, scale, self.window,
                                scratch=ctx.rt.scratch)
                 return
-        ops.attention_plain(q, ctx.meta, kv, out, self.nq, self.nkv, self.hd, self.kernel_scale, self.window)
+        ops.attention_plain(q, ctx.meta, kv, out, self.nq, self.nkv, self.hd, scale, self.window)

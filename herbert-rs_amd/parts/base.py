@@ -159,6 +159,9 @@ class StepContext:
     # (x's address, alpha): a block whose norm comes after the sum has left, for the next such block, the
     # rows that its first part reads and alpha times x where that part adds
     pending_post: Any = None
+    # (x's address, delta, factors): a pre-norm block with scaled branches has left its last branch for the next
+    # such block's first norm to add to x (x += factors * delta, a factor a channel)
+    pending_scaled: Any = None
 
     def adds_to(self, x):
         """False if x are the context's fresh rows (the part's product stores), True if it has to add."""

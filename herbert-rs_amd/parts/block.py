@@ -9,13 +9,31 @@ take x as it is, and each norm comes after its sum.
 "prenorm": x += mixer(norm_input(x)); x += feed_forward(norm_post_mixer(x)), the
 arrangement of the reference's two-norm layer
 (crates/backends/backend_common/src/generic_layer.rs:1149-1151, 1234-1236,
-1246-1248, 1272-1274).
+1246-1248, 1272-1274). With `branch_scale` (not in the reference) each branch is multiplied, channel by
+channel, by a learned factor before it joins x, and the layer may have no feed-forward.
 """
 import torch
 
 from ..kernels import ops
+from ..weights import TensorNeed
 from .base import Part
 from .registry import register
+
+
+class ChannelScale(Part):
+    """A learned factor a channel on a branch's output, before the branch joins the residual stream."""
+    graph_safe = True
+
+    def __init__(self, size, weight):
+        self.size = int(size)
+        self.weight_name = weight
+        self.w = None
+
+    def tensor_needs(self):
+        return {self.weight_name: TensorNeed((self.size,), "scale")}
+
+    def load(self, tensors, rt):
+        self.w = rt.weight(tensors[self.weight_name], matrix=False)
 
 
 @register("block", "prenorm")
@@ -24,22 +42,79 @@ class PreNormBlock(Part):
 
     norm_roles = ("input", "post_mixer")
 
-    def __init__(self, mixer, feed_forward, norms):
+    def __init__(self, mixer, feed_forward, norms, branch_scale=None):
+        """branch_scale: None, or {"size": the model's width, "mixer": tensor name, "feed_forward": tensor name}:
+        each branch times a stored factor a channel before the sum. Such a block's parts add to float32 rows
+        of their own; the kernel of the norm that follows adds them, scaled, to x on its way (the last
+        branch of a layer is left for the next layer's first norm, if that is such a block too). Only such
+        a block may do without a feed-forward."""
         self.mixer = mixer
         self.feed_forward = feed_forward
         self.norms = norms
-        missing = [r for r in self.norm_roles if r not in norms]
+        self.scales = None
+        if branch_scale is not None:
+            self.scales = {"mixer": ChannelScale(branch_scale["size"], branch_scale["mixer"])}
+            if feed_forward is not None:
+                self.scales["feed_forward"] = ChannelScale(branch_scale["size"], branch_scale["feed_forward"])
+        elif feed_forward is None:
+            raise ValueError("prenorm block: only a block with scaled branches may do without a feed-forward")
+        missing = [r for r in self.norm_roles[:1 if feed_forward is None else 2] if r not in norms]
         if missing:
             raise ValueError(f"prenorm block needs norms {missing}")
+        if self.scales is not None:
+            for role in self.norm_roles:
+                if role in norms and not getattr(norms[role], "takes_scaled_sum", False):
+                    raise ValueError("prenorm block: with scaled branches its norms must take a scaled sum on")
 
     def parts(self):
-        return [self.norms["input"], self.mixer, self.norms["post_mixer"], self.feed_forward]
+        parts = [self.norms["input"], self.mixer]
+        if self.feed_forward is not None:
+            parts += [self.norms["post_mixer"], self.feed_forward]
+        if self.scales is not None:
+            parts += list(self.scales.values())
+        return parts
 
     def first_norm(self):
         """The norm that the residual stream meets first in this block."""
         return self.norms["input"]
 
+    def takes_scaled_sum(self):
+        """True if this block's first norm adds the scaled branch that the block before left (ctx.pending_scaled)."""
+        return self.scales is not None
+
+    def _forward_scaled(self, ctx, x):
+        branch = ctx.rt.buffer("branch_sum", tuple(x.shape), torch.float32)
+        pending, ctx.pending_scaled = ctx.pending_scaled, None
+        if pending is not None and pending[0] == x.data_ptr():
+            h = self.norms["input"].forward(ctx, x, delta=pending[1], factors=pending[2])
+        else:
+            h = self.norms["input"].forward(ctx, x)
+        steps = [(self.mixer, self.scales["mixer"])]
+        if self.feed_forward is not None:
+            steps.append((self.feed_forward, self.scales["feed_forward"]))
+        for i, (part, scale) in enumerate(steps):
+            ctx.handed = ctx.norm_ahead = ctx.left = None
+            # a part that can store its rows instead of adding them says so and finds the rows in ctx.fresh_rows;
+            # for any other the rows are cleared first
+            if getattr(part, "stores_fresh_rows", False):
+                ctx.fresh_rows = branch
+            else:
+                ops.fill_u32(branch, 0)
+            part.forward(ctx, h, branch)
+            ctx.fresh_rows = None
+            if i + 1 < len(steps):
+                h = self.norms["post_mixer"].forward(ctx, x, delta=branch, factors=scale.w)
+                continue
+            nxt = ctx.next_block
+            if isinstance(nxt, PreNormBlock) and nxt.takes_scaled_sum():
+                ctx.pending_scaled = (x.data_ptr(), branch, scale.w)
+            else:
+                ops.rmsnorm_scaled_sum(x, branch, scale.w, None, None, 0.0)
+
     def forward(self, ctx, x):
+        if self.scales is not None:
+            self._forward_scaled(ctx, x)
+            return
         after = ctx.norm_after_block
         self._run(ctx, x, self.norms["input"], self.mixer, (self.norms["post_mixer"], ctx.entry))
         self._run(ctx, x, self.norms["post_mixer"], self.feed_forward, after)

@@ -1,4 +1,5 @@
-"""Dense feed-forwards without biases. "swiglu": down(silu(gate(y)) * up(y)). "squared_relu": down(max(up(y), 0)^2).
+"""Dense feed-forwards without biases. "swiglu": down(f(gate(y)) * up(y)) with f = silu, or with `activation="gelu_tanh"`
+the tanh form of gelu. "squared_relu": down(max(up(y), 0)^2).
 
 crates/backends/backend_common/src/generic_mlp.rs:83-96 and kernels.rs:676-687
 of the reference; gate and up are one fused matrix here so that the activations
@@ -16,9 +17,13 @@ from .registry import register
 @register("feed_forward", "swiglu")
 class SwiGLU(Part):
     graph_safe = True
+    stores_fresh_rows = True     # its last product stores into rows that hold nothing yet (StepContext.adds_to)
 
-    def __init__(self, hidden_size, intermediate_size, names, shared=None):
-        """names: dict with gate, up, down -> tensor names."""
+    def __init__(self, hidden_size, intermediate_size, names, shared=None, activation="silu"):
+        """names: dict with gate, up, down -> tensor names. activation: "silu" or "gelu_tanh" (on the gate)."""
+        if activation not in ops.GLU_ACTIVATIONS:
+            raise ValueError(f"the gated unit's activation is one of {sorted(ops.GLU_ACTIVATIONS)}, not {activation!r}")
+        self.activation = activation
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
         self.names = dict(names)
@@ -36,7 +41,7 @@ class SwiGLU(Part):
         gate, up = rt.weight(tensors[n["gate"]]), rt.weight(tensors[n["up"]])
         # bfloat16 with sizes the MFMA kernel takes: gate and up rows interleaved so that the
         # product's epilogue applies silu(gate) * up and the float32 [T, 2I] never exists
-        self.fused_epilogue = (rt.dtype == torch.bfloat16 and self.intermediate_size % 16 == 0
+        self.fused_epilogue = (self.activation == "silu" and rt.dtype == torch.bfloat16 and self.intermediate_size % 16 == 0
                                and self.hidden_size % 32 == 0 and mfma.gemm_supported(
                                    gate[:1], gate, swiglu=True))
         if self.fused_epilogue:
@@ -70,9 +75,10 @@ class SwiGLU(Part):
         else:
             gu = rt.buffer("gate_up", (T, 2 * self.intermediate_size), torch.float32)
             self.gate_up.forward(y, gu)
-            ops.swiglu(gu, act)
-        left = ctx.leave_norm(self.down, x)
-        self.down.forward(act, x, accumulate=True, leave=None if left is None else left.leave())
+            ops.swiglu(gu, act, self.activation)
+        adds = ctx.adds_to(x)
+        left = ctx.leave_norm(self.down, x) if adds else None
+        self.down.forward(act, x, accumulate=adds, leave=None if left is None else left.leave())
 
 
 @register("feed_forward", "squared_relu")

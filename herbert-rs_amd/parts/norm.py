@@ -17,6 +17,7 @@ def _around_zero(shape, gen, device, std, norm_std):
 class RMSNorm(Part):
     graph_safe = True
     hands_on = True      # y = x * w / rms(x): a product may apply the 1 / rms to its sums instead (NormedRows)
+    takes_scaled_sum = True     # forward(..., delta=, factors=) first adds factors * delta to x (a factor a channel)
 
     def __init__(self, size, eps, weight, offset=0.0):
         """offset: added to the stored weight (1 for weights stored as offsets from one)."""
@@ -36,10 +37,17 @@ class RMSNorm(Part):
         if self.offset:
             self.w = (self.w + self.offset).contiguous()
 
-    def forward(self, ctx, x, rows=None, name="normed"):
+    def forward(self, ctx, x, rows=None, name="normed", delta=None, factors=None):
+        """delta f32 [T, size] with factors f32 [size]: x becomes x + factors * delta first, in place, and that
+        sum is normed, in one kernel (no rows then)."""
         n = x.shape[0] if rows is None else rows.shape[0]
         y = ctx.rt.buffer(name, (n, self.size))
-        ops.rmsnorm(x, self.w, y, self.eps, rows)
+        if delta is not None:
+            if rows is not None:
+                raise ValueError("rmsnorm: rows are not gathered while a sum is added")
+            ops.rmsnorm_scaled_sum(x, delta, factors, self.w, y, self.eps)
+        else:
+            ops.rmsnorm(x, self.w, y, self.eps, rows)
         return y
 
 

@@ -87,3 +87,49 @@ class RotaryHalfSplit(Part):
     def rotation_rates(self):
         """(inv_freq float32 [rotary_dims / 2] on the GPU, rotary_dims): entry i turns by position * inv_freq[i]."""
         return self.rates, self.rotary_dims
+
+
+@register("position", "rope_pairs")
+class RotaryPairs(Part):
+    """Rotation of neighbouring pairs: entries 2i and 2i + 1 of a head's first `rotary_dims` turn by
+    position x theta^(-2i / rotary_dims). No tables: a mixer's kernel takes the rates (float64) and computes
+    a position's angle, its sine and its cosine itself, so no table bounds the positions.
+    scaling = (factor, low, high, original): a rate whose wavelength 2 pi / rate lies beyond original / low is
+    divided by factor, one under original / high stays, and between the two, with
+    s = (original / wavelength - low) / (high - low), the rate is (1 - s) rate / factor + s rate."""
+    graph_safe = True
+
+    def __init__(self, theta, rotary_dims, scaling=None):
+        if rotary_dims % 2 or rotary_dims <= 0:
+            raise ValueError("rotary_dims must be even and positive")
+        self.theta, self.rotary_dims = float(theta), int(rotary_dims)
+        self.scaling = None if scaling is None else tuple(float(v) for v in scaling)
+        self.rates = None
+
+    def pair_rates_host(self):
+        rates = []
+        for i in range(self.rotary_dims // 2):
+            rate = self.theta ** (-2.0 * i / self.rotary_dims)
+            if self.scaling is not None:
+                factor, low, high, original = self.scaling
+                wavelength = 2.0 * math.pi / rate
+                if wavelength > original / low:
+                    rate = rate / factor
+                elif wavelength >= original / high:
+                    s = (original / wavelength - low) / (high - low)
+                    rate = (1.0 - s) * rate / factor + s * rate
+            rates.append(rate)
+        return rates
+
+    def load(self, tensors, rt):
+        self.rates = torch.tensor(self.pair_rates_host(), dtype=torch.float64).to(rt.device)
+
+    def rotation(self):
+        return None
+
+    def rotation_rates(self):
+        return None
+
+    def pair_rates(self):
+        """(rates float64 [rotary_dims / 2] on the GPU, rotary_dims)."""
+        return self.rates, self.rotary_dims
