@@ -66,6 +66,15 @@ __device__ __forceinline__ float max_with_other_half(float v) {
 }
 
 #define RESCALE_LOG2 8.0f
+
+// A sink: a score without key or value that the softmax's denominator of a head also holds, exp(sink),
+// unscaled, once. It joins the sum at the end, in the units of the reference m that the sum was taken
+// against (raw scores; c = scale * log2 e): 2^(sink * log2 e - m c). m lags behind the largest score by
+// at most RESCALE_LOG2, so the share neither overflows nor loses digits that count; an infinite share
+// (a sink far above every score) gives the output 0, its limit.
+__device__ __forceinline__ float sink_share(float sink, float m, float c) {
+    return fast_exp2(sink * 1.4426950408889634f - (m == -INFINITY ? 0.f : m * c));
+}
 template <bool MASKED>
 __device__ __forceinline__ void softmax_page(f32x16 st[2], int g2, int page0, int lo, int hi, float c,
                                              float& m, float& l, float& corr, bf16x8 pb[2][2]) {
@@ -268,7 +277,7 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache
                     const int* __restrict__ tile_seq, const int* __restrict__ tile_row0,
                     const int* __restrict__ tile_rows, const int* __restrict__ positions,
                     const int* __restrict__ slots, const int* __restrict__ page_table, int max_pages, int nq,
-                    int nkv, float c, int window, int per_tile) {
+                    int nkv, float c, int window, int per_tile, const float* __restrict__ sinks) {
     constexpr int KCH = HD / 8;                   // 16-byte chunks of a key row
     constexpr int KRPB = 128 / HD > 0 ? 128 / HD : 1;   // key rows in 256 bytes
     constexpr int KROWS = 512 / HD;               // key rows a load instruction brings (1 KB)
@@ -433,8 +442,10 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache
         for (int d = 0; d < HD / 32; ++d)
 #pragma unroll
             for (int i = 0; i < 16; ++i) oacc[d][i] = oacc[d][i] * a0 + hand[(2 + d * 16 + i) * 64] * a1;
+        m = mm;
     }
     l += __shfl_xor(l, 32, 64);
+    if (sinks) l += sink_share(sinks[h], m, c);
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     bf16* orow = out + ((size_t)(row0 + c32) * nq + h) * HD;
 #pragma unroll
@@ -464,7 +475,8 @@ attn_prefill_long_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
                          const int* __restrict__ tile_seq, const int* __restrict__ tile_row0,
                          const int* __restrict__ tile_rows, const int* __restrict__ positions,
                          const int* __restrict__ slots, const int* __restrict__ page_table, int max_pages,
-                         int nq, int nkv, float c, int window, int per_tile) {
+                         int nq, int nkv, float c, int window, int per_tile,
+                         const float* __restrict__ sinks) {
     constexpr int KCH = HD / 8;
     constexpr int KRPB = 128 / HD > 0 ? 128 / HD : 1;
     constexpr int KROWS = 512 / HD;
@@ -608,6 +620,7 @@ attn_prefill_long_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
     hb_wait_vmcnt<0>();          // nothing of this workgroup's is in flight when it ends
     if (!active || c32 >= rows) return;
     l += __shfl_xor(l, 32, 64);
+    if (sinks) l += sink_share(sinks[h], m, c);
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     bf16* orow = out + ((size_t)(row0 + c32) * nq + h) * HD;
 #pragma unroll
@@ -651,7 +664,7 @@ attn_decode_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_cache, bf16*
                    const int* __restrict__ context_lens, const int* __restrict__ slots,
                    const int* __restrict__ page_table, int max_pages, int nq, int nkv, float c, int window,
                    int pages_per_split, DecodeFusion fu, bf16* __restrict__ out,
-                   const int* __restrict__ ranges, int n_seqs) {
+                   const int* __restrict__ ranges, int n_seqs, const float* __restrict__ sinks) {
     // ranges == null: the grid is (sequence, kv head, range), every sequence cut into gridDim.z
     // ranges of pages_per_split pages (those past a sequence's end hold nothing).
     // ranges != null (sequences of unequal lengths): the grid is (1, kv head, item);
@@ -891,6 +904,7 @@ attn_decode_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_cache, bf16*
     if (out) {
         // one range a sequence: nothing to merge, the output is O / l (zeros if no key was visible)
         if (c32 < G) {
+            if (sinks) l += sink_share(sinks[kvh * G + c32], m, c);
             const float inv = l > 0.f ? 1.0f / l : 0.f;
             bf16* dst = out + ((size_t)b * nq + kvh * G + c32) * HD;
 #pragma unroll
@@ -930,7 +944,8 @@ attn_decode_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_cache, bf16*
 template <int HD>
 __global__ void __launch_bounds__(256)
 attn_decode_merge_kernel(const float* __restrict__ partial_o, const float* __restrict__ partial_ml,
-                         bf16* __restrict__ out, int splits, float c, const int* __restrict__ ranges, int nq) {
+                         bf16* __restrict__ out, int splits, float c, const int* __restrict__ ranges, int nq,
+                         const float* __restrict__ sinks) {
     // thread = (group of ranges, 4 consecutive d): it adds up the weighted partial sums of the ranges
     // g, g + GROUPS, ... once the first wave has worked out the weights; the groups are then added
     // in order through LDS. (Asking for the partial sums before the weights are known gains nothing:
@@ -971,6 +986,7 @@ attn_decode_merge_kernel(const float* __restrict__ partial_o, const float* __res
             for (int off = 32; off > 0; off >>= 1) term += __shfl_xor(term, off, 64);
             denom += term;
         }
+        if (sinks) denom += sink_share(sinks[bh % nq], M, c);      // once a (sequence, head), whatever the ranges
         if (tid == 0) s_inv = denom > 0.f ? 1.0f / denom : 0.f;
     }
     __syncthreads();
@@ -1000,7 +1016,8 @@ extern "C" int hb_attn_prefill_mfma(const void* q, const void* k_cache, const vo
                                     const int* tile_seq, const int* tile_row0, const int* tile_rows,
                                     int num_tiles, const int* positions, const int* slots,
                                     const int* page_table, int max_pages, int page_size, int nq, int nkv,
-                                    int hd, float scale, int window, int tile_height, hipStream_t stream) {
+                                    int hd, float scale, int window, int tile_height, const float* sinks,
+                                    hipStream_t stream) {
     HB_REQUIRE(num_tiles > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attn_prefill: bad sizes");
     HB_REQUIRE(page_size == PAGE, "attn_prefill: pages must hold %d tokens", PAGE);
     HB_REQUIRE(window >= 0, "attn_prefill: bad window");
@@ -1025,7 +1042,7 @@ extern "C" int hb_attn_prefill_mfma(const void* q, const void* k_cache, const vo
         }                                                                                                \
         KERNEL<HDV><<<total, 512, lds, stream>>>((const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache, \
                                                  (bf16*)out, tile_seq, tile_row0, tile_rows, positions, slots, \
-                                                 page_table, max_pages, nq, nkv, c, window, per_tile);   \
+                                                 page_table, max_pages, nq, nkv, c, window, per_tile, sinks); \
     } while (0)
     if (tile_height == 64) {
         if (hd == 32) LAUNCH_PREFILL(attn_prefill_long_kernel, 32);
@@ -1052,7 +1069,7 @@ extern "C" int hb_attn_decode_mfma(const void* q, void* k_cache, void* v_cache, 
                                    int pages_per_split, const float* qkv, const float* q_norm_w,
                                    const float* k_norm_w, const float* cos_t, const float* sin_t, float eps,
                                    int write_kv, int qkv_slices, size_t slice_stride, const int* ranges,
-                                   float q_temp_coef, int q_temp_every, hipStream_t stream) {
+                                   float q_temp_coef, int q_temp_every, const float* sinks, hipStream_t stream) {
     // ranges != null: see attn_decode_kernel; `splits` is then the number of items of the grid (the
     // partial results are [nq, splits]), pages_per_split is not read
     HB_REQUIRE(!ranges || (B >= 2 && splits >= 2 && window == 0),
@@ -1073,7 +1090,8 @@ extern "C" int hb_attn_decode_mfma(const void* q, void* k_cache, void* v_cache, 
     HB_REQUIRE(qkv || q, "attn_decode: neither q nor the projection rows are given");
     HB_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "attn_decode: cos and sin tables come together");
 #define DECODE_ARGS(QPTR) QPTR, (bf16*)k_cache, (bf16*)v_cache, partial_o, partial_ml, context_lens, slots, \
-                          page_table, max_pages, nq, nkv, c, window, pages_per_split, fu, direct, ranges, B
+                          page_table, max_pages, nq, nkv, c, window, pages_per_split, fu, direct, ranges, B, \
+                          direct ? sinks : nullptr
 #define LAUNCH_DECODE(HDV) do {                                                                          \
     if (qkv)                                                                                             \
         attn_decode_kernel<HDV, true><<<grid, 64, 0, stream>>>(DECODE_ARGS(nullptr));                    \
@@ -1092,7 +1110,7 @@ extern "C" int hb_attn_decode_mfma(const void* q, void* k_cache, void* v_cache, 
 #undef DECODE_ARGS
     HB_CHECK_LAUNCH("attn_decode");
     if (!direct) {
-#define LAUNCH_MERGE(HDV) attn_decode_merge_kernel<HDV><<<B * nq, 256, 0, stream>>>(partial_o, partial_ml, (bf16*)out, splits, c, ranges, nq)
+#define LAUNCH_MERGE(HDV) attn_decode_merge_kernel<HDV><<<B * nq, 256, 0, stream>>>(partial_o, partial_ml, (bf16*)out, splits, c, ranges, nq, sinks)
         if (hd == 32) LAUNCH_MERGE(32);
         else if (hd == 64) LAUNCH_MERGE(64);
         else LAUNCH_MERGE(128);

@@ -387,9 +387,9 @@ def gemm_swiglu(a, w_interleaved, out, packed=False, norm=None, tile=0, row_scal
 
 
 lib.register_signatures("attention_mfma", {
-    "hb_attn_prefill_mfma": [_P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P],
+    "hb_attn_prefill_mfma": [_P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P],
     "hb_attn_decode_mfma": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I,
-                            _P, _P, _P, _P, _P, _F, _I, _I, ctypes.c_size_t, _P, _F, _I, _P],
+                            _P, _P, _P, _P, _P, _F, _I, _I, ctypes.c_size_t, _P, _F, _I, _P, _P],
 })
 
 ATTENTION_HEAD_DIMS = (32, 64, 128)
@@ -583,14 +583,15 @@ def attention_decode_fused(qkv, q_norm_w, k_norm_w, cos, sin, meta, kv, out, nq,
              window, splits, per, src, None if q_norm_w is None else q_norm_w.data_ptr(),
              None if k_norm_w is None else k_norm_w.data_ptr(), None if cos is None else cos.data_ptr(),
              None if sin is None else sin.data_ptr(), float(eps), 1, n_slices, stride,
-             None if ranges is None else ranges.data_ptr(), coef, every, _stream())
+             None if ranges is None else ranges.data_ptr(), coef, every, None, _stream())
 
 
 DEFERRED_SLICES = (2, 4, 8)     # numbers of slices of the projection that the decode kernel adds up itself
 
 
-def attention(q, meta, kv, out, nq, nkv, hd, scale, window, tile_height=None, scratch=None):
+def attention(q, meta, kv, out, nq, nkv, hd, scale, window, tile_height=None, scratch=None, sinks=None):
     """Causal (and windowed) attention of the step's tokens over their slots' pages.
+    sinks f32 [nq]: the softmax's denominator of head h also holds exp(sinks[h]), once, without key or value.
     One token a sequence: the split decode kernel; otherwise one of the two tiled prompt kernels
     (tile_height 32 or 64 asks for one by name; None: the host's choice, see _prefill_tile_height)."""
     T = q.shape[0]
@@ -604,6 +605,9 @@ def attention(q, meta, kv, out, nq, nkv, hd, scale, window, tile_height=None, sc
     if not attention_supported(q, kv, nq, nkv, hd):
         raise BackendError(f"attention_mfma refuses head_dim {hd} with {nq}/{nkv} heads")
     window = int(window or 0)
+    if sinks is not None:
+        _check(sinks, "sinks", torch.float32, (nq,))
+    sinks_ptr = None if sinks is None else sinks.data_ptr()
     if meta.max_new == 1:
         if T != meta.num_seqs:
             raise BackendError("decode attention needs one token for each sequence")
@@ -619,7 +623,7 @@ def attention(q, meta, kv, out, nq, nkv, hd, scale, window, tile_height=None, sc
                  out.data_ptr(), po.data_ptr(), pml.data_ptr(), meta.context_lens.data_ptr(),
                  meta.slots.data_ptr(), kv.page_table.data_ptr(), kv.page_table.shape[1], kv.page_size,
                  T, nq, nkv, hd, float(scale), window, splits, per, None, None, None, None, None, 0.0, 0, 1, 0,
-                 None if ranges is None else ranges.data_ptr(), 0.0, 0, _stream())
+                 None if ranges is None else ranges.data_ptr(), 0.0, 0, sinks_ptr, _stream())
         return
     _check(meta.positions, "positions", torch.int32, (T,))
     height = tile_height or _prefill_tile_height(meta, nkv, nq // nkv)
@@ -629,4 +633,4 @@ def attention(q, meta, kv, out, nq, nkv, hd, scale, window, tile_height=None, sc
     lib.call("attention_mfma", "hb_attn_prefill_mfma", q.data_ptr(), kv.k.data_ptr(), kv.v.data_ptr(),
              out.data_ptr(), tile_seq.data_ptr(), tile_row0.data_ptr(), tile_rows.data_ptr(), n_tiles,
              meta.positions.data_ptr(), meta.slots.data_ptr(), kv.page_table.data_ptr(),
-             kv.page_table.shape[1], kv.page_size, nq, nkv, hd, float(scale), window, height, _stream())
+             kv.page_table.shape[1], kv.page_size, nq, nkv, hd, float(scale), window, height, sinks_ptr, _stream())

@@ -322,12 +322,9 @@ class Attention(Part):
 
     def attend(self, ctx, q, kv, out):
         scale = self.scale if self.prepared else self.kernel_scale
-        if self.sink_w is not None:
-            ops.attention_plain(q, ctx.meta, kv, out, self.nq, self.nkv, self.hd, scale, self.window, sinks=self.sink_w)
-            return
         if q.dtype == torch.bfloat16:
             if mfma.attention_supported(q, kv, self.nq, self.nkv, self.hd):
                 mfma.attention(q, ctx.meta, kv, out, self.nq, self.nkv, self.hd, scale, self.window,
-                               scratch=ctx.rt.scratch)
+                               scratch=ctx.rt.scratch, sinks=self.sink_w)
                 return
-        ops.attention_plain(q, ctx.meta, kv, out, self.nq, self.nkv, self.hd, scale, self.window)
+        ops.attention_plain(q, ctx.meta, kv, out, self.nq, self.nkv, self.hd, scale, self.window, sinks=self.sink_w)
