@@ -99,8 +99,8 @@ def _w():
 
 
 def _f():
-    # F: for keys far back and long memories: sharper scores than a random model's (the tests scale the norms'
-    #    weights), decays near one
+    # F: for keys far back and long memories: scores three times as sharp as a random model's usual ones (the
+    #    scale), and the tests set the decays of both recurrences near one
     layers = [rglru(128, 4, 3),
               parallel(left(4, 2, 64, 64, 0.4, 3, rot(64, 1000.0, (4.0, 1.0, 4.0, 128))), right(2, 32, 32, 8.0, 16), ff=256)]
     return model(384, 128, layers, eps=1e-6, loop=(0, 2, 2))
