@@ -21,7 +21,7 @@ step is what the generation loop does for a token: the step function (a HIP-grap
 greedy choice on the GPU, and the chosen tokens read by the host, which as in that loop reads
 the tokens of a step while the next step, fed from the GPU, already runs.
 
-`--workload vipalorn|modasun --size small|medium|wide` measures one of the other designs instead (random weights at
+`--workload vipalorn|modasun|mefatar --size small|medium|wide` measures one of the other designs instead (random weights at
 sizes that resemble a real model's layers) beside the closest other model at equal size, through the generation
 loop; the default workload and its JSON line stay as they are.
 """
@@ -187,9 +187,28 @@ def modasun_configs(size):
     return mod, family_configs(size)[0]
 
 
+def mefatar_configs(size):
+    """(Mefatar config dict, Modasun config dict) of one size: two layers with the real-gated recurrent unit (as wide
+    as the model, a block of gates a head, four taps) to one layer with the two mixers side by side (the softmax
+    attention with four taps, the whole head rotated with slowed wavelengths, a sink and a gate; the linear
+    attention with half the heads, keys of half the size and a decay through a middle of a sixteenth of the
+    width), every layer with a dense feed-forward as wide as the experts that a token of the other model uses
+    together; and the Modasun model of the same width, depth and heads."""
+    W, L, H, D, V, rank, rot, E, top, ff, vocab = FAMILY_SIZES[size]
+    mlp = {"kind": "dense", "ff": top * ff}
+    unit = {"type": "rglru", "mixer": {"width": W, "blocks": H, "conv": 4}, "mlp": mlp}
+    left = {"heads": H, "kv_heads": H // 2, "dim": D, "vdim": V, "scale": D ** -0.5, "conv": 4,
+            "rot": {"dims": D, "base": 10000.0, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    right = {"heads": H // 2, "dim": D // 2, "vdim": V, "tau": 16.0, "rank": W // 16}
+    sides = {"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": mlp}
+    layers = [sides if i % 3 == 2 else unit for i in range(L)]
+    mef = {"architecture": "Mefatar", "vocab": vocab, "width": W, "layers": layers, "norm": {"eps": 1e-6}}
+    return mef, modasun_configs(size)[0]
+
+
 def run_family(args, names=("vipalorn", "qwen3"), configs=family_configs):
     """Prompt and decode throughput of a design at one size (random weights) beside the closest other model at
-    equal size (Vipalorn beside the dense Qwen3 decoder, Modasun beside Vipalorn), both through the generation
+    equal size (Vipalorn beside the dense Qwen3 decoder, Modasun beside Vipalorn, Mefatar beside Modasun), both through the generation
     loop: prompts of 512 and 2,048 tokens alone, and batches of 1, 8 and 32 sequences of 1,024 prompt tokens
     decoding `--steps` tokens each."""
     import torch
@@ -260,9 +279,9 @@ def main():
     ap.add_argument("--no-sweep", action="store_true", help="time the full context only, not 512 and the mean")
     ap.add_argument("--no-long", action="store_true",
                     help="skip the further sizes and lengths (contexts of 16 K and 32 K, batch 128 and 256, long prompts)")
-    ap.add_argument("--size", default="medium", choices=sorted(FAMILY_SIZES), help="layer sizes of --workload vipalorn and --workload modasun")
-    ap.add_argument("--workload", default="headline", choices=["headline", "qwen3-1.7b", "qwen3-32b", "vipalorn", "modasun"],
-                    help="headline: BASELINE.json configs[2]; qwen3-*: configs[3] and configs[4]; vipalorn, modasun: "
+    ap.add_argument("--size", default="medium", choices=sorted(FAMILY_SIZES), help="layer sizes of --workload vipalorn, modasun and mefatar")
+    ap.add_argument("--workload", default="headline", choices=["headline", "qwen3-1.7b", "qwen3-32b", "vipalorn", "modasun", "mefatar"],
+                    help="headline: BASELINE.json configs[2]; qwen3-*: configs[3] and configs[4]; vipalorn, modasun, mefatar: "
                          "that design at --size beside the closest other model at equal size")
     ap.add_argument("--prefill-tokens", type=int, default=2048, help="length of the prompt of the prefill figure")
     ap.add_argument("--prefill-chunk", type=int, default=0,
@@ -286,6 +305,9 @@ def main():
         return 0
     if args.workload == "modasun":
         print(json.dumps(run_family(args, names=("modasun", "vipalorn"), configs=modasun_configs)))
+        return 0
+    if args.workload == "mefatar":
+        print(json.dumps(run_family(args, names=("mefatar", "modasun"), configs=mefatar_configs)))
         return 0
     if args.workload != "headline":
         print(json.dumps(run_workload(args, 3 if args.workload == "qwen3-1.7b" else 4,
