@@ -709,12 +709,62 @@ __global__ void rmsnorm_scaled_sum_kernel(float* x, const float* __restrict__ de
     for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = hb_from_float<TOut>(in[i] * inv * w[i]);
 }
 
+// The same for rows of up to 4096 numbers in steps of four: a thread keeps its up to sixteen sums in registers
+// between the two passes (16-byte loads and stores), so that the second pass waits for no memory.
+template <class TOut>
+__global__ void __launch_bounds__(256)
+rmsnorm_scaled_sum_held_kernel(float* x, const float* __restrict__ delta, const float* __restrict__ ls,
+                               const float* __restrict__ w, TOut* y, int H, float eps) {
+    __shared__ float red[16];
+    const size_t row = (size_t)blockIdx.x * H;
+    const int quads = H / 4;
+    float4 held[4];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int q = threadIdx.x + j * 256;
+        if (q < quads) {
+            const float4 a = *(const float4*)(x + row + 4 * q), d = *(const float4*)(delta + row + 4 * q);
+            const float4 f = *(const float4*)(ls + 4 * q);
+            float4 v;
+            v.x = fmaf(f.x, d.x, a.x), v.y = fmaf(f.y, d.y, a.y), v.z = fmaf(f.z, d.z, a.z), v.w = fmaf(f.w, d.w, a.w);
+            *(float4*)(x + row + 4 * q) = v;
+            held[j] = v;
+            ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+        }
+    }
+    if (y == nullptr) return;
+    ss = hb_block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int q = threadIdx.x + j * 256;
+        if (q < quads) {
+            const float4 g = *(const float4*)(w + 4 * q);
+            TOut* out = y + row + 4 * q;
+            out[0] = hb_from_float<TOut>(held[j].x * inv * g.x);
+            out[1] = hb_from_float<TOut>(held[j].y * inv * g.y);
+            out[2] = hb_from_float<TOut>(held[j].z * inv * g.z);
+            out[3] = hb_from_float<TOut>(held[j].w * inv * g.w);
+        }
+    }
+}
+
 extern "C" int hb_rmsnorm_scaled_sum(float* x, const float* delta, const float* ls, const float* w, void* y,
                                      int y_dtype, int R, int H, float eps, hipStream_t stream) {
     HB_REQUIRE(R > 0 && H > 0, "rmsnorm: empty input (R=%d, H=%d)", R, H);
     HB_REQUIRE(delta != nullptr && ls != nullptr, "rmsnorm: a scaled sum needs its rows and its factors");
     HB_REQUIRE(y == nullptr || w != nullptr, "rmsnorm: a norm needs its weight");
     HB_REQUIRE(y_dtype == HB_F32 || y_dtype == HB_BF16, "rmsnorm: unknown output dtype %d", y_dtype);
+    if (H % 4 == 0 && H >= 1024 && H <= 4096 && (uintptr_t)x % 16 == 0 && (uintptr_t)delta % 16 == 0 &&
+        (uintptr_t)ls % 16 == 0 && (w == nullptr || (uintptr_t)w % 16 == 0)) {
+        if (y_dtype == HB_F32)
+            rmsnorm_scaled_sum_held_kernel<float><<<R, 256, 0, stream>>>(x, delta, ls, w, (float*)y, H, eps);
+        else
+            rmsnorm_scaled_sum_held_kernel<bf16><<<R, 256, 0, stream>>>(x, delta, ls, w, (bf16*)y, H, eps);
+        HB_CHECK_LAUNCH("rmsnorm_scaled_sum_held");
+        return 0;
+    }
     const int threads = H >= 1024 ? 256 : H >= 256 ? 128 : 64;
     if (y_dtype == HB_F32)
         rmsnorm_scaled_sum_kernel<float><<<R, threads, 0, stream>>>(x, delta, ls, w, (float*)y, H, eps);
@@ -770,7 +820,7 @@ extern "C" int hb_normed_pair(const float* a, const float* wa, float ca, const f
 //   norm (weights null: none): all queries of the token are divided by their common root mean square and
 //     multiplied by q_norm_w [nq x dim], the keys likewise with k_norm_w [nkv x dim];
 //   rotation (rates null: none): entries 2i and 2i + 1 of the first rot_dims of every query and key head turn
-//     by position x rates[i]; rates are float64 and so are the angle, its sine and its cosine;
+//     by position x rates[i]; rates and the angle are float64, sine and cosine float32 of the angle reduced to [-pi, pi];
 //   q_out [T, nq x hd], key pages [page, kv head, token, hd], value pages [page, kv head, hd, token]: heads
 //     are kept at size hd >= max(dim, vdim), the entries beyond a head's own size are zeros.
 template <class TQ, class TC>
@@ -813,10 +863,15 @@ filter_norm_rotate_write_kernel(const float* __restrict__ proj, int ld, const fl
     }
     if (rates != nullptr) {
         for (int i = tid; i < rot_dims / 2; i += 256) {
-            double s, c;
-            sincos((double)pos * rates[i], &s, &c);
-            cs[2 * i] = (float)c;
-            cs[2 * i + 1] = (float)s;
+            // the angle and its reduction to [-pi, pi] in float64 (a few operations), sine and cosine of the reduced
+            // angle in float32: a float64 sincos costs as much as the rest of the kernel
+            const double a = (double)pos * rates[i];
+            const double turns = rint(a * 0.15915494309189535);
+            const double r = fma(-turns, 1.2246467991473532e-16 * 2.0, fma(-turns, 6.283185307179586, a));
+            float s, c;
+            sincosf((float)r, &s, &c);
+            cs[2 * i] = c;
+            cs[2 * i + 1] = s;
         }
     }
     sq = hb_block_sum(sq, red);           // (its barriers also publish `filtered` and the angles)

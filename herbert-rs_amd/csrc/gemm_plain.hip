@@ -130,7 +130,12 @@ static void launch(const void* A, const void* W, void* C, int M, int N, int K, i
 #define FEW_ROWS_K 1024
 __global__ void __launch_bounds__(HB_WAVE)
 gemm_few_rows_kernel(const float* __restrict__ A, const bf16* __restrict__ W, float* __restrict__ C, int M, int N,
-                     int K, int lda, int ldw, int ldc, DecayEpilogue ep) {
+                     int K, int lda, int ldw, int ldc, DecayEpilogue ep, size_t batch_a = 0, size_t batch_w = 0,
+                     size_t batch_c = 0) {
+    // (blockIdx.z: one of a batch of products whose operands lie batch_* elements apart)
+    A += blockIdx.z * batch_a;
+    W += blockIdx.z * batch_w;
+    C += blockIdx.z * batch_c;
     __shared__ __attribute__((aligned(16))) float rows_of_a[FEW_ROWS_M * FEW_ROWS_K];
     const int lane = threadIdx.x;
     const int n = blockIdx.x * 16 + lane / 4;
@@ -255,6 +260,14 @@ extern "C" int hb_gemm_plain_batched(const void* A, int a_dtype, const void* W, 
     HB_REQUIRE(M > 0 && N > 0 && K > 0 && batch > 0, "gemm: empty problem (M=%d, N=%d, K=%d, batch=%d)", M, N, K, batch);
     HB_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gemm: a row stride is smaller than its row");
     HB_REQUIRE((M + TILE_M - 1) / TILE_M <= 65535 && batch <= 65535, "gemm: M=%d or batch=%d exceeds the grid", M, batch);
+    // few rows (one token a sequence) with a short k: the kernel made for them, a product of the batch a grid's layer
+    if (few_rows_takes(A, a_dtype, W, w_dtype, c_dtype, M, K, lda, ldw, 0) && batch_a % 4 == 0 && batch_w % 8 == 0) {
+        gemm_few_rows_kernel<<<dim3((N + 15) / 16, (M + FEW_ROWS_M - 1) / FEW_ROWS_M, batch), HB_WAVE, 0, stream>>>(
+            (const float*)A, (const bf16*)W, (float*)C, M, N, K, lda, ldw, ldc, DecayEpilogue{nullptr, nullptr, 1, 0.f},
+            batch_a, batch_w, batch_c);
+        HB_CHECK_LAUNCH("gemm_few_rows_batched");
+        return 0;
+    }
     const int key = a_dtype * 4 + w_dtype * 2 + c_dtype;
 #define HB_BATCHED(TA, TW, TC) launch<TA, TW, TC>(A, W, C, M, N, K, lda, ldw, ldc, 0, stream, batch, batch_a, batch_w, batch_c)
     switch (key) {

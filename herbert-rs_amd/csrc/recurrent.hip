@@ -195,11 +195,86 @@ __global__ void lru_scan_kernel(const float* __restrict__ ug, const float* __res
     *S_mem = S;
 }
 
+// The same recurrence for long portions. S_t = a_t S_(t-1) + b_t is a chain, but its pieces compose: over a run
+// of tokens the state leaves as A S + B with A the product of the run's decays and B the run's walk from zero. A
+// workgroup is SEGS waves on 64 channels; a sequence's tokens are cut into SEGS runs. Every wave but the last first
+// walks its run from zero (A, B into LDS); then each wave takes the sequence's state through the runs before its
+// own (at most SEGS - 1 multiply-adds) and walks its run again from there, now storing the outputs. The chain is
+// two runs long instead of the whole portion; the decays and inputs are computed twice (their loads come from
+// the cache the second time). The result differs from the one-wave walk by float32 rounding (the runs' edges).
+template <class TOut, int SEGS>
+__global__ void __launch_bounds__(64 * SEGS)
+lru_scan_runs_kernel(const float* __restrict__ ug, const float* __restrict__ gates, const float* __restrict__ rb,
+                     const float* __restrict__ ib, const float* __restrict__ lam, float rate, float* __restrict__ state,
+                     const int* __restrict__ seq_starts, const int* __restrict__ slots, TOut* __restrict__ y, int W, int bw) {
+    __shared__ float sA[SEGS][64], sB[SEGS][64];
+    const int seq = blockIdx.x;
+    const int lane = threadIdx.x & 63, seg = threadIdx.x >> 6;
+    const int c = blockIdx.y * 64 + lane;
+    const bool live = c < W;
+    const int cc = live ? c : 0;
+    const int gc = (cc / bw) * 2 * bw + cc % bw;
+    const int first = seq_starts[seq], n = seq_starts[seq + 1] - first;
+    const int per = (n + SEGS - 1) / SEGS;
+    const int t0 = first + min(seg * per, n), t1 = first + min((seg + 1) * per, n);
+    const float z = lam[cc];
+    const float step = -rate * (z > 20.f ? z : log1pf(expf(z)));
+    const float rbc = rb[cc], ibc = ib[cc];
+    auto decay_and_input = [&](int t, float& a, float& in) {
+        const float r = 1.0f / (1.0f + expf(-(gates[(size_t)t * 2 * W + gc] + rbc)));
+        const float i = 1.0f / (1.0f + expf(-(gates[(size_t)t * 2 * W + gc + bw] + ibc)));
+        const float log_a = step * r;
+        a = expf(log_a);
+        in = sqrtf(-expm1f(2.0f * log_a)) * i * ug[(size_t)t * 2 * W + cc];
+    };
+    float A = 1.f, B = 0.f;
+    if (live && seg < SEGS - 1) {
+#pragma unroll 4
+        for (int t = t0; t < t1; ++t) {
+            float a, in;
+            decay_and_input(t, a, in);
+            B = fmaf(a, B, in);
+            A *= a;
+        }
+    }
+    sA[seg][lane] = A;
+    sB[seg][lane] = B;
+    __syncthreads();
+    float* S_mem = state + (size_t)slots[seq] * W + cc;
+    float S = live ? *S_mem : 0.f;
+    for (int k = 0; k < seg; ++k) S = fmaf(sA[k][lane], S, sB[k][lane]);
+    if (!live) return;
+#pragma unroll 4
+    for (int t = t0; t < t1; ++t) {
+        float a, in;
+        decay_and_input(t, a, in);
+        S = fmaf(a, S, in);
+        y[(size_t)t * W + c] = hb_from_float<TOut>(S * ug[(size_t)t * 2 * W + W + c]);
+    }
+    if (seg == SEGS - 1) *S_mem = S;
+}
+
+// longest: the most tokens that one sequence of the step brings (the host knows it); portions of LRU_RUNS_FROM
+// tokens or more take the kernel that cuts them into runs.
+#define LRU_RUNS_FROM 128
+#define LRU_RUNS 16
+
 extern "C" int hb_lru_scan(const float* ug, const float* gates, const float* rb, const float* ib, const float* lam,
                            float rate, float* state, const int* seq_starts, const int* slots, void* y, int y_dtype,
-                           int B, int W, int bw, hipStream_t stream) {
+                           int B, int W, int bw, int longest, hipStream_t stream) {
     HB_REQUIRE(B > 0 && W > 0 && B <= 65535, "recurrent unit: empty input or too many sequences for the grid");
     HB_REQUIRE(bw > 0 && W % bw == 0, "recurrent unit: %d channels in blocks of %d", W, bw);
+    if (longest >= LRU_RUNS_FROM) {
+        const dim3 grid(B, (W + 63) / 64);
+        if (y_dtype == HB_F32)
+            lru_scan_runs_kernel<float, LRU_RUNS><<<grid, 64 * LRU_RUNS, 0, stream>>>(ug, gates, rb, ib, lam, rate, state, seq_starts, slots, (float*)y, W, bw);
+        else if (y_dtype == HB_BF16)
+            lru_scan_runs_kernel<bf16, LRU_RUNS><<<grid, 64 * LRU_RUNS, 0, stream>>>(ug, gates, rb, ib, lam, rate, state, seq_starts, slots, (bf16*)y, W, bw);
+        else
+            HB_REQUIRE(false, "recurrent unit: unknown output dtype %d", y_dtype);
+        HB_CHECK_LAUNCH("lru_scan_runs");
+        return 0;
+    }
     const int threads = W >= 4096 ? 256 : 64;          // (few channels: more, smaller workgroups over the CUs)
     const dim3 grid(B, (W + threads - 1) / threads);
     if (y_dtype == HB_F32)

@@ -26,7 +26,7 @@ def rand(*shape, seed=0, scale=1.0):
 
 
 # ---------------------------------------------------------------- sums, norms, the gated unit
-@pytest.mark.parametrize("H", [24, 72, 1536])
+@pytest.mark.parametrize("H", [24, 72, 1536, 2052, 4096])
 def test_scaled_sum_then_norm(H):
     x, d, f, w = rand(7, H, seed=1, scale=2.0), rand(7, H, seed=2), 0.5 + 0.3 * rand(H, seed=3), 1 + 0.1 * rand(H, seed=4)
     want_x = x + f * d
@@ -75,13 +75,22 @@ def unit_reference(proj, W, bx, by, taps, fb, r_w, r_b, i_w, i_b, lam):
     return u.float(), g.float(), (plain.gated_recurrence(u, r, i, lam) * g).float()
 
 
-@pytest.mark.parametrize("W,blocks,K", [(8, 8, 1), (96, 3, 4), (40, 1, 2), (256, 4, 3), (192, 6, 4)])
-def test_recurrent_unit_whole_in_portions_and_token_by_token(W, blocks, K):
+@pytest.mark.parametrize("W,blocks,K,lengths,all_cuts", [
+    (8, 8, 1, [41, 3, 18], ([], [1, 2, 3, 9, 17, 40], list(range(1, 41)))),
+    (96, 3, 4, [41, 3, 18], ([], [1, 2, 3, 9, 17, 40], list(range(1, 41)))),
+    (40, 1, 2, [41, 3, 18], ([], [1, 2, 3, 9, 17, 40], list(range(1, 41)))),
+    (256, 4, 3, [41, 3, 18], ([], [1, 2, 3, 9, 17, 40], list(range(1, 41)))),
+    (192, 6, 4, [41, 3, 18], ([], [1, 2, 3, 9, 17, 40], list(range(1, 41)))),
+    # portions of 128 tokens and more are walked as sixteen runs side by side: lengths that the runs divide and
+    # do not, a sequence shorter than the number of runs beside a long one, a long portion after a short one
+    (96, 3, 4, [333, 5, 140], ([], [130], [2, 131, 132, 260])),
+    (72, 2, 2, [128, 128, 1], ([], [127])),
+])
+def test_recurrent_unit_whole_in_portions_and_token_by_token(W, blocks, K, lengths, all_cuts):
     """Portions shorter than the filter's taps, single tokens, sequences of unequal lengths in one step, slots
     that the pass before used; rates from memories of a few tokens to ones that outlast the sequence."""
     b = W // blocks
     ld = 2 * W + 5
-    lengths = [41, 3, 18]
     bx, by, fb = 0.3 * rand(W, seed=1), 0.3 * rand(W, seed=2), 0.2 * rand(W, seed=3)
     taps = 1.0 / K + 0.3 * rand(W, K, seed=4)
     r_w, i_w = rand(blocks, b, b, seed=5) / b ** 0.5, rand(blocks, b, b, seed=6) / b ** 0.5
@@ -90,10 +99,10 @@ def test_recurrent_unit_whole_in_portions_and_token_by_token(W, blocks, K):
     projs = [rand(n, ld, seed=10 + i, scale=1.5) for i, n in enumerate(lengths)]
     refs = [unit_reference(p, W, bx, by, taps, fb, r_w, r_b, i_w, i_b, lam) for p in projs]
     gate_w = torch.cat([r_w, i_w], 1).contiguous().to(DEV)                # [blocks, 2 b, b]
-    cache = Cache({0: (StateNeed((W,)), StateNeed((max(K - 1, 1), W)))}, 64 * 8, 4096, torch.float32, DEV, max_slots=4)
+    cache = Cache({0: (StateNeed((W,)), StateNeed((max(K - 1, 1), W)))}, 64 * 16, 4096, torch.float32, DEV, max_slots=4)
     state, conv_state = cache.state_views(0)
     g = lambda t: t.reshape(-1).contiguous().to(DEV)
-    for cuts in ([], [1, 2, 3, 9, 17, 40], list(range(1, 41))):
+    for cuts in all_cuts:
         slots = [cache.alloc_slot() for _ in lengths]
         got = [[] for _ in lengths]
         edges = sorted(set([0] + cuts + [max(lengths)]))
