@@ -816,23 +816,26 @@ extern "C" int hb_normed_pair(const float* a, const float* wa, float ca, const f
 // C columns. One workgroup a token:
 //   filter (taps [C, K], K >= 1; null: none): y[c] = sum_j taps[c, j] * in[t - (K - 1) + j, c], the inputs
 //     before the step's first row from the slot's state [K - 1, C] (zeros in a fresh slot); the state is
-//     moved on by a kernel of its own afterwards (hb_filter_state in the module of the recurrent mixers);
+//     moved on by a kernel of its own afterwards (hb_filter_state in the module of the recurrent mixers), or
+//     here where every sequence brings one token;
 //   norm (weights null: none): all queries of the token are divided by their common root mean square and
 //     multiplied by q_norm_w [nq x dim], the keys likewise with k_norm_w [nkv x dim];
 //   rotation (rates null: none): entries 2i and 2i + 1 of the first rot_dims of every query and key head turn
 //     by position x rates[i]; rates and the angle are float64, sine and cosine float32 of the angle reduced to [-pi, pi];
 //   q_out [T, nq x hd], key pages [page, kv head, token, hd], value pages [page, kv head, hd, token]: heads
 //     are kept at size hd >= max(dim, vdim), the entries beyond a head's own size are zeros.
-template <class TQ, class TC>
+// TK: the taps' count where it is 2, 3 or 4 (the filter's loop is then unrolled and all of a thread's loads of an
+// iteration are in flight together), 0: any count.
+template <class TQ, class TC, int TK>
 __global__ void __launch_bounds__(256)
 filter_norm_rotate_write_kernel(const float* __restrict__ proj, int ld, const float* __restrict__ taps, int K,
-                                const float* __restrict__ filter_state, const float* __restrict__ q_norm_w,
+                                float* __restrict__ filter_state, const float* __restrict__ q_norm_w,
                                 const float* __restrict__ k_norm_w, const double* __restrict__ rates, int rot_dims,
                                 const int* __restrict__ positions, const int* __restrict__ seq_of,
                                 const int* __restrict__ seq_starts, const int* __restrict__ slots,
                                 const int* __restrict__ page_table, int max_pages, int page_size,
                                 TQ* __restrict__ q_out, TC* __restrict__ k_cache, TC* __restrict__ v_cache, int nq,
-                                int nkv, int dim, int vdim, int hd, float eps) {
+                                int nkv, int dim, int vdim, int hd, float eps, int moves_state) {
     extern __shared__ float filtered[];           // [C] the token's channels, then [rot_dims] cosines and sines
     __shared__ float red[16];
     const int t = blockIdx.x, tid = threadIdx.x;
@@ -843,23 +846,64 @@ filter_norm_rotate_write_kernel(const float* __restrict__ proj, int ld, const fl
     const int at = t - first;
     const int slot = slots[seq];
     const int pos = positions[t];
-    const float* state = filter_state + (size_t)slot * (K > 1 ? K - 1 : 1) * C;
+    float* state = filter_state + (size_t)slot * (K > 1 ? K - 1 : 1) * C;
+    const int page = page_table[(size_t)slot * max_pages + pos / page_size];       // (asked for early: used last)
+    const int in_page = pos % page_size;
     float sq = 0.f, sk = 0.f;
-    for (int c = tid; c < C; c += 256) {
-        float y;
+    // eight channels a thread at a time, so that a tap's eight loads are in flight together (one channel after
+    // the other, every load would wait for the one before: the taps' count is not known when this is compiled)
+    for (int c0 = tid; c0 < C; c0 += 8 * 256) {
+        float y[8], wn[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            // the norm's weight of the channel, loaded here beside the filter's operands: the loops that store the
+            // heads then read LDS only and wait for no memory
+            const int c = c0 + u * 256;
+            y[u] = 0.f;
+            wn[u] = 1.f;
+            if (c < QD) { if (q_norm_w) wn[u] = q_norm_w[c]; }
+            else if (c < QD + KD) { if (k_norm_w) wn[u] = k_norm_w[c - QD]; }
+        }
         if (taps == nullptr) {
-            y = proj[(size_t)t * ld + c];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int c = c0 + u * 256;
+                if (c < C) y[u] = proj[(size_t)t * ld + c];
+            }
         } else {
-            y = 0.f;
-            for (int j = 0; j < K; ++j) {
-                const int s = at - (K - 1) + j;
-                const float v = s >= 0 ? proj[(size_t)(first + s) * ld + c] : state[(size_t)(K - 1 + s) * C + c];
-                y = fmaf(taps[(size_t)c * K + j], v, y);
+            const int taps_n = TK > 0 ? TK : K;
+#pragma unroll
+            for (int j = 0; j < taps_n; ++j) {
+                const int s = at - (taps_n - 1) + j;
+                const float* row = s >= 0 ? proj + (size_t)(first + s) * ld : state + (size_t)(taps_n - 1 + s) * C;
+                float v[8], w[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int c = c0 + u * 256;
+                    v[u] = c < C ? row[c] : 0.f;
+                    w[u] = c < C ? taps[(size_t)c * taps_n + j] : 0.f;
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) y[u] = fmaf(w[u], v[u], y[u]);
+                // one token a sequence: this thread is the only reader of its channels' kept inputs and moves
+                // them on itself (each takes the place of the one before it, the last the token's own input)
+                if (moves_state && j > 0) {
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) {
+                        const int c = c0 + u * 256;
+                        if (c < C) state[(size_t)(j - 1) * C + c] = v[u];
+                    }
+                }
             }
         }
-        filtered[c] = y;
-        if (c < QD) sq = fmaf(y, y, sq);
-        else if (c < QD + KD) sk = fmaf(y, y, sk);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int c = c0 + u * 256;
+            if (c >= C) continue;
+            filtered[c] = y[u] * wn[u];
+            if (c < QD) sq = fmaf(y[u], y[u], sq);
+            else if (c < QD + KD) sk = fmaf(y[u], y[u], sk);
+        }
     }
     if (rates != nullptr) {
         for (int i = tid; i < rot_dims / 2; i += 256) {
@@ -880,9 +924,9 @@ filter_norm_rotate_write_kernel(const float* __restrict__ proj, int ld, const fl
     const float inv_k = k_norm_w ? 1.0f / sqrtf(sk / (float)KD + eps) : 1.0f;
     const int rd = rates != nullptr ? rot_dims : 0;
     // one entry of a query or key head after norm and rotation; c0: the head's first channel
-    auto turned = [&](int c0, int d, const float* w, float inv) {
+    auto turned = [&](int c0, int d, float inv) {
         if (d >= dim) return 0.f;
-        auto normed = [&](int e) { return w ? filtered[c0 + e] * inv * w[c0 + e] : filtered[c0 + e]; };
+        auto normed = [&](int e) { return filtered[c0 + e] * inv; };        // (the weight is in `filtered` already)
         if (d >= rd) return normed(d);
         const int i = d >> 1;
         const float u = normed(2 * i), v = normed(2 * i + 1);
@@ -891,27 +935,24 @@ filter_norm_rotate_write_kernel(const float* __restrict__ proj, int ld, const fl
     };
     for (int idx = tid; idx < nq * hd; idx += 256) {
         const int h = idx / hd, d = idx - h * hd;
-        q_out[(size_t)t * nq * hd + idx] = hb_from_float<TQ>(turned(h * dim, d, q_norm_w, inv_q));
+        q_out[(size_t)t * nq * hd + idx] = hb_from_float<TQ>(turned(h * dim, d, inv_q));
     }
-    const int page = page_table[(size_t)slot * max_pages + pos / page_size];
-    const int in_page = pos % page_size;
     for (int idx = tid; idx < nkv * hd; idx += 256) {
         const int g = idx / hd, d = idx - g * hd;
-        const float* kw = k_norm_w ? k_norm_w - QD : nullptr;       // (indexed by the channel within the row)
         const size_t base = ((size_t)page * nkv + g) * page_size * hd;
-        k_cache[base + (size_t)in_page * hd + d] = hb_from_float<TC>(turned(QD + g * dim, d, kw, inv_k));
+        k_cache[base + (size_t)in_page * hd + d] = hb_from_float<TC>(turned(QD + g * dim, d, inv_k));
         const float v = d < vdim ? filtered[QD + KD + g * vdim + d] : 0.f;
         v_cache[base + (size_t)d * page_size + in_page] = hb_from_float<TC>(v);
     }
 }
 
-extern "C" int hb_filter_norm_rotate_write(const float* proj, int ld, const float* taps, int K, const float* filter_state,
+extern "C" int hb_filter_norm_rotate_write(const float* proj, int ld, const float* taps, int K, float* filter_state,
                                            const float* q_norm_w, const float* k_norm_w, const double* rates,
                                            int rot_dims, const int* positions, const int* seq_of,
                                            const int* seq_starts, const int* slots, const int* page_table,
                                            int max_pages, int page_size, void* q_out, void* k_cache, void* v_cache,
                                            int dtype, int T, int nq, int nkv, int dim, int vdim, int hd, float eps,
-                                           hipStream_t stream) {
+                                           int longest, hipStream_t stream) {
     HB_REQUIRE(T > 0 && nq > 0 && nkv > 0 && dim > 0 && vdim > 0, "filtered attention: empty input");
     HB_REQUIRE(hd >= dim && hd >= vdim, "filtered attention: heads kept at %d cannot hold %d and %d", hd, dim, vdim);
     const long long C = (long long)(nq + nkv) * dim + (long long)nkv * vdim;
@@ -923,16 +964,29 @@ extern "C" int hb_filter_norm_rotate_write(const float* proj, int ld, const floa
     const size_t lds = ((size_t)C + (rates ? rot_dims : 0)) * sizeof(float);
     HB_REQUIRE(lds <= 60 * 1024, "filtered attention: %lld channels a token do not fit the kernel's LDS", C);
     if (taps == nullptr) K = 0;
+    // longest: the most tokens that a sequence of the step brings; at one the kernel moves the filter's state on
+    // itself, otherwise hb_filter_state does so afterwards
+    const int moves_state = longest == 1 && K > 1;
+#define HB_FNRW(TQ, TC, TK)                                                                                              \
+    filter_norm_rotate_write_kernel<TQ, TC, TK><<<T, 256, lds, stream>>>(                                                  \
+        proj, ld, taps, K, filter_state, q_norm_w, k_norm_w, rates, rot_dims, positions, seq_of, seq_starts, slots,       \
+        page_table, max_pages, page_size, (TQ*)q_out, (TC*)k_cache, (TC*)v_cache, nq, nkv, dim, vdim, hd, eps,   \
+        moves_state)
+#define HB_FNRW_TAPS(TQ, TC)                                                                                             \
+    do {                                                                                                                 \
+        if (K == 4) HB_FNRW(TQ, TC, 4);                                                                                  \
+        else if (K == 3) HB_FNRW(TQ, TC, 3);                                                                             \
+        else if (K == 2) HB_FNRW(TQ, TC, 2);                                                                             \
+        else HB_FNRW(TQ, TC, 0);                                                                                         \
+    } while (0)
     if (dtype == HB_F32)
-        filter_norm_rotate_write_kernel<float, float><<<T, 256, lds, stream>>>(
-            proj, ld, taps, K, filter_state, q_norm_w, k_norm_w, rates, rot_dims, positions, seq_of, seq_starts, slots,
-            page_table, max_pages, page_size, (float*)q_out, (float*)k_cache, (float*)v_cache, nq, nkv, dim, vdim, hd, eps);
+        HB_FNRW_TAPS(float, float);
     else if (dtype == HB_BF16)
-        filter_norm_rotate_write_kernel<bf16, bf16><<<T, 256, lds, stream>>>(
-            proj, ld, taps, K, filter_state, q_norm_w, k_norm_w, rates, rot_dims, positions, seq_of, seq_starts, slots,
-            page_table, max_pages, page_size, (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, nq, nkv, dim, vdim, hd, eps);
+        HB_FNRW_TAPS(bf16, bf16);
     else
         HB_REQUIRE(false, "filtered attention: unknown dtype %d", dtype);
+#undef HB_FNRW_TAPS
+#undef HB_FNRW
     HB_CHECK_LAUNCH("filter_norm_rotate_write");
     return 0;
 }

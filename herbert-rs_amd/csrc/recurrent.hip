@@ -120,22 +120,33 @@ __device__ __forceinline__ float lru_gelu_tanh(float z) {
 
 __global__ void lru_inputs_kernel(const float* __restrict__ proj, int ld, const float* __restrict__ bx,
                                   const float* __restrict__ by, const float* __restrict__ taps,
-                                  const float* __restrict__ fb, const float* __restrict__ conv_state,
+                                  const float* __restrict__ fb, float* __restrict__ conv_state,
                                   const int* __restrict__ seq_of, const int* __restrict__ seq_starts,
-                                  const int* __restrict__ slots, float* __restrict__ out, int W, int K) {
+                                  const int* __restrict__ slots, float* __restrict__ out, int W, int K,
+                                  int moves_state) {
     const int t = blockIdx.x;
     const int c = blockIdx.y * blockDim.x + threadIdx.x;
     if (c >= W) return;
     const int seq = seq_of[t];
     const int first = seq_starts[seq];
     const int at = t - first;
-    const float* state = conv_state + (size_t)slots[seq] * (K > 1 ? K - 1 : 1) * W;
+    float* state = conv_state + (size_t)slots[seq] * (K > 1 ? K - 1 : 1) * W;
     const float b = bx[c];
     float acc = fb ? fb[c] : 0.f;
-    for (int j = 0; j < K; ++j) {
-        const int s = at - (K - 1) + j;
-        const float v = s >= 0 ? proj[(size_t)(first + s) * ld + c] + b : state[(size_t)(K - 1 + s) * W + c];
-        acc = fmaf(taps[(size_t)c * K + j], v, acc);
+    if (moves_state) {
+        // one token a sequence: this thread is the only reader of its channel's K - 1 kept inputs, so it also
+        // moves them on (each takes the next one's place, the last the token's own input)
+        for (int j = 0; j < K; ++j) {
+            const float v = j < K - 1 ? state[(size_t)j * W + c] : proj[(size_t)t * ld + c] + b;
+            acc = fmaf(taps[(size_t)c * K + j], v, acc);
+            if (j > 0) state[(size_t)(j - 1) * W + c] = v;
+        }
+    } else {
+        for (int j = 0; j < K; ++j) {
+            const int s = at - (K - 1) + j;
+            const float v = s >= 0 ? proj[(size_t)(first + s) * ld + c] + b : state[(size_t)(K - 1 + s) * W + c];
+            acc = fmaf(taps[(size_t)c * K + j], v, acc);
+        }
     }
     out[(size_t)t * 2 * W + c] = acc;
     out[(size_t)t * 2 * W + W + c] = lru_gelu_tanh(proj[(size_t)t * ld + W + c] + by[c]);
@@ -143,14 +154,16 @@ __global__ void lru_inputs_kernel(const float* __restrict__ proj, int ld, const 
 
 extern "C" int hb_lru_inputs(const float* proj, int ld, const float* bx, const float* by, const float* taps,
                              const float* fb, float* conv_state, const int* seq_of, const int* seq_starts,
-                             const int* slots, float* out, int T, int B, int W, int K, hipStream_t stream) {
+                             const int* slots, float* out, int T, int B, int W, int K, int longest, hipStream_t stream) {
     HB_REQUIRE(T > 0 && B > 0 && W > 0 && ld >= 2 * W, "recurrent unit: empty input or rows of %d for 2 x %d channels", ld, W);
     HB_REQUIRE(K >= 1 && K <= HB_MAX_TAPS, "recurrent unit: %d taps, the kernel takes 1 to %d", K, HB_MAX_TAPS);
     HB_REQUIRE((W + 255) / 256 <= 65535 && B <= 65535, "recurrent unit: too many channels or sequences for the grid");
+    // one token a sequence at most (longest: the most that a sequence of the step brings): the kernel moves the state on itself
+    const int moves_state = longest == 1 && K > 1;
     lru_inputs_kernel<<<dim3(T, (W + 255) / 256), 256, 0, stream>>>(proj, ld, bx, by, taps, fb, conv_state, seq_of,
-                                                                    seq_starts, slots, out, W, K);
+                                                                    seq_starts, slots, out, W, K, moves_state);
     HB_CHECK_LAUNCH("lru_inputs");
-    if (K > 1) {
+    if (K > 1 && !moves_state) {
         conv_state_kernel<<<dim3(B, (W + 255) / 256), 256, 0, stream>>>(proj, ld, conv_state, seq_starts, slots, W, K, bx);
         HB_CHECK_LAUNCH("lru_filter_state");
     }

@@ -28,7 +28,7 @@ SIGNATURES = {
         "hb_rmsnorm_scaled_sum": [_P, _P, _P, _P, _P, _I, _I, _I, _F, _P],
         "hb_normed_pair": [_P, _P, _F, _P, _P, _F, _P, _I, _I, _F, _I, _P],
         "hb_filter_norm_rotate_write": [_P, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P,
-                                        _I, _I, _I, _I, _I, _I, _I, _F, _P],
+                                        _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
         "hb_gate_heads": [_P, _I, _P, _I, _I, _P, _I, _I, _I, _I, _P],
         "hb_fill_u32": [_P, _U32, _SZ, _P],
         "hb_layernorm": [_P, _P, _F, _P, _P, _I, _P, _I, _I, _F, _P],
@@ -45,7 +45,7 @@ SIGNATURES = {
         "hb_conv_silu": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _I, _P],
         "hb_gated_delta": [_P, _I, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
         "hb_filter_state": [_P, _I, _P, _P, _P, _I, _I, _I, _P, _P],
-        "hb_lru_inputs": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+        "hb_lru_inputs": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
         "hb_lru_scan": [_P, _P, _P, _P, _P, _F, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
         "hb_gated_head_norm": [_P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _P],
         "hb_channel_decay": [_P, _I, _P, _P, _P, _I, _I, _I, _P],

@@ -527,7 +527,8 @@ def filter_norm_rotate_write(proj, taps, filter_state, q_norm_w, k_norm_w, rates
     no filter), queries and keys each normed over the whole projection (weights [nq x dim], [nkv x dim]; None:
     no norm), neighbouring pairs of the first rot_dims entries of every head turned by position x rates (f64
     [rot_dims / 2]; None: no rotation); q to q_out [T, nq x hd], keys and values to the token's page, heads kept
-    at hd with zeros beyond their own size. The filter's state is moved on by recurrent.filter_state."""
+    at hd with zeros beyond their own size. The filter's state is moved on too: by the kernel itself where every
+    sequence brings one token (meta.max_new), by the filter-state kernel afterwards otherwise."""
     T, ld = proj.shape
     C = (nq + nkv) * dim + nkv * vdim
     _check(proj, "proj", torch.float32, (T, ld))
@@ -554,7 +555,12 @@ def filter_norm_rotate_write(proj, taps, filter_state, q_norm_w, k_norm_w, rates
              _ptr(filter_state) if K > 1 else None, _ptr(q_norm_w), _ptr(k_norm_w), _ptr(rates), int(rot_dims),
              meta.positions.data_ptr(), meta.seq_of.data_ptr(), meta.seq_starts.data_ptr(), meta.slots.data_ptr(),
              cache.page_table.data_ptr(), cache.page_table.shape[1], cache.page_size, q_out.data_ptr(),
-             cache.k.data_ptr(), cache.v.data_ptr(), dtype_code(q_out), T, nq, nkv, dim, vdim, hd, float(eps), _stream())
+             cache.k.data_ptr(), cache.v.data_ptr(), dtype_code(q_out), T, nq, nkv, dim, vdim, hd, float(eps),
+             int(meta.max_new), _stream())
+    if K > 1 and meta.max_new != 1:
+        _check(meta.slots, "slots", torch.int32, (meta.num_seqs,))
+        lib.call("recurrent", "hb_filter_state", proj.data_ptr(), ld, filter_state.data_ptr(), meta.seq_starts.data_ptr(),
+                 meta.slots.data_ptr(), meta.num_seqs, C, K, None, _stream())
 
 
 def gate_heads(attn, gate_rows, g_off, out, nq, hd, vdim):

@@ -154,7 +154,8 @@ def lru_inputs(proj, bx, by, taps, filter_bias, conv_state, meta, out):
         raise BackendError(f"recurrent unit: rows of {ld} for 2 x {W} channels, {K} taps")
     lib.call("recurrent", "hb_lru_inputs", proj.data_ptr(), ld, bx.data_ptr(), by.data_ptr(), taps.data_ptr(),
              None if filter_bias is None else filter_bias.data_ptr(), conv_state.data_ptr(), meta.seq_of.data_ptr(),
-             meta.seq_starts.data_ptr(), meta.slots.data_ptr(), out.data_ptr(), T, meta.num_seqs, W, K, _stream())
+             meta.seq_starts.data_ptr(), meta.slots.data_ptr(), out.data_ptr(), T, meta.num_seqs, W, K, int(meta.max_new),
+             _stream())
 
 
 def lru_scan(ug, gates, r_bias, i_bias, lam, rate, state, meta, out, block):

@@ -220,8 +220,6 @@ class Attention(Part):
         rates, rot_dims = self.position.pair_rates() if hasattr(self.position, "pair_rates") else (None, 0)
         ops.filter_norm_rotate_write(proj, self.taps_w, state, self.q_norm_w, self.k_norm_w, rates, rot_dims, ctx.meta,
                                      kv, q, self.nq, self.nkv, self.dim, self.vdim, self.hd, self.eps)
-        if self.taps > 1:
-            recurrent.filter_state(proj, state, ctx.meta, self.channels, self.taps)
         attn = rt.buffer("attn", (T, self.q_dim))
         self.attend(ctx, q, kv, attn)
         # the heads leave at their own size, each entry times its gate

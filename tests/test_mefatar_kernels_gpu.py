@@ -250,8 +250,6 @@ def test_prepared_attention_with_a_sink_and_a_far_key(nq, nkv, dim, vdim, K, rot
             T = p.shape[0]
             q = torch.empty(T, nq * hd, dtype=dtype, device=DEV)
             ops.filter_norm_rotate_write(p, g(taps), state, g(qw), g(kw), rates, rot_dims, meta, kv, q, nq, nkv, dim, vdim, hd, eps)
-            if K > 1:
-                recurrent.filter_state(p, state, meta, C, K)
             attn = torch.full_like(q, 9.0)
             if dtype == torch.bfloat16 and mfma.attention_supported(q, kv, nq, nkv, hd):
                 mfma.attention(q, meta, kv, attn, nq, nkv, hd, scale, 0, sinks=g(sinks))
