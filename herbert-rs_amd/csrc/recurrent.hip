@@ -208,17 +208,36 @@ __global__ void lru_scan_kernel(const float* __restrict__ ug, const float* __res
     *S_mem = S;
 }
 
-// The same recurrence for long portions. S_t = a_t S_(t-1) + b_t is a chain, but its pieces compose: over a run
-// of tokens the state leaves as A S + B with A the product of the run's decays and B the run's walk from zero. A
-// workgroup is SEGS waves on 64 channels; a sequence's tokens are cut into SEGS runs. Every wave but the last first
-// walks its run from zero (A, B into LDS); then each wave takes the sequence's state through the runs before its
-// own (at most SEGS - 1 multiply-adds) and walks its run again from there, now storing the outputs. The chain is
-// two runs long instead of the whole portion; the decays and inputs are computed twice (their loads come from
-// the cache the second time). The result differs from the one-wave walk by float32 rounding (the runs' edges).
+// The same recurrence for long portions, in two kernels. The first, one thread a (token, channel), turns the gates'
+// pre-activations into the decay a and the input b = sqrt(1 - a^2) i u where they lie (`gates` is overwritten: r_pre's
+// place takes a, i_pre's place b): the exponentials and the root are most of the arithmetic, and here they fill
+// the chip. The second walks S_t = a_t S_(t-1) + b_t, a chain, but one whose pieces compose: over a run of tokens
+// the state leaves as A S + B with A the product of the run's decays and B the run's walk from zero. A workgroup
+// is SEGS waves on 64 channels; a sequence's tokens are cut into SEGS runs. Every wave but the last first walks
+// its run from zero (A, B into LDS); then each wave takes the sequence's state through the runs before its own (at
+// most SEGS - 1 multiply-adds) and walks its run again from there, now storing the outputs. The chain is two runs
+// long instead of the whole portion. The result differs from the one-wave walk by float32 rounding (the runs' edges).
+__global__ void lru_decay_input_kernel(const float* __restrict__ ug, float* __restrict__ gates,
+                                       const float* __restrict__ rb, const float* __restrict__ ib,
+                                       const float* __restrict__ lam, float rate, int W, int bw, size_t total) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const size_t t = idx / W;
+    const int c = (int)(idx - t * W);
+    const int gc = (c / bw) * 2 * bw + c % bw;
+    float* row = gates + t * 2 * W;
+    const float z = lam[c];
+    const float step = -rate * (z > 20.f ? z : log1pf(expf(z)));
+    const float r = 1.0f / (1.0f + expf(-(row[gc] + rb[c])));
+    const float i = 1.0f / (1.0f + expf(-(row[gc + bw] + ib[c])));
+    const float log_a = step * r;
+    row[gc] = expf(log_a);
+    row[gc + bw] = sqrtf(-expm1f(2.0f * log_a)) * i * ug[t * 2 * W + c];
+}
+
 template <class TOut, int SEGS>
 __global__ void __launch_bounds__(64 * SEGS)
-lru_scan_runs_kernel(const float* __restrict__ ug, const float* __restrict__ gates, const float* __restrict__ rb,
-                     const float* __restrict__ ib, const float* __restrict__ lam, float rate, float* __restrict__ state,
+lru_scan_runs_kernel(const float* __restrict__ ug, const float* __restrict__ ab, float* __restrict__ state,
                      const int* __restrict__ seq_starts, const int* __restrict__ slots, TOut* __restrict__ y, int W, int bw) {
     __shared__ float sA[SEGS][64], sB[SEGS][64];
     const int seq = blockIdx.x;
@@ -230,22 +249,11 @@ lru_scan_runs_kernel(const float* __restrict__ ug, const float* __restrict__ gat
     const int first = seq_starts[seq], n = seq_starts[seq + 1] - first;
     const int per = (n + SEGS - 1) / SEGS;
     const int t0 = first + min(seg * per, n), t1 = first + min((seg + 1) * per, n);
-    const float z = lam[cc];
-    const float step = -rate * (z > 20.f ? z : log1pf(expf(z)));
-    const float rbc = rb[cc], ibc = ib[cc];
-    auto decay_and_input = [&](int t, float& a, float& in) {
-        const float r = 1.0f / (1.0f + expf(-(gates[(size_t)t * 2 * W + gc] + rbc)));
-        const float i = 1.0f / (1.0f + expf(-(gates[(size_t)t * 2 * W + gc + bw] + ibc)));
-        const float log_a = step * r;
-        a = expf(log_a);
-        in = sqrtf(-expm1f(2.0f * log_a)) * i * ug[(size_t)t * 2 * W + cc];
-    };
     float A = 1.f, B = 0.f;
     if (live && seg < SEGS - 1) {
-#pragma unroll 4
+#pragma unroll 8
         for (int t = t0; t < t1; ++t) {
-            float a, in;
-            decay_and_input(t, a, in);
+            const float a = ab[(size_t)t * 2 * W + gc], in = ab[(size_t)t * 2 * W + gc + bw];
             B = fmaf(a, B, in);
             A *= a;
         }
@@ -257,10 +265,9 @@ lru_scan_runs_kernel(const float* __restrict__ ug, const float* __restrict__ gat
     float S = live ? *S_mem : 0.f;
     for (int k = 0; k < seg; ++k) S = fmaf(sA[k][lane], S, sB[k][lane]);
     if (!live) return;
-#pragma unroll 4
+#pragma unroll 8
     for (int t = t0; t < t1; ++t) {
-        float a, in;
-        decay_and_input(t, a, in);
+        const float a = ab[(size_t)t * 2 * W + gc], in = ab[(size_t)t * 2 * W + gc + bw];
         S = fmaf(a, S, in);
         y[(size_t)t * W + c] = hb_from_float<TOut>(S * ug[(size_t)t * 2 * W + W + c]);
     }
@@ -272,17 +279,21 @@ lru_scan_runs_kernel(const float* __restrict__ ug, const float* __restrict__ gat
 #define LRU_RUNS_FROM 128
 #define LRU_RUNS 16
 
-extern "C" int hb_lru_scan(const float* ug, const float* gates, const float* rb, const float* ib, const float* lam,
+extern "C" int hb_lru_scan(const float* ug, float* gates, const float* rb, const float* ib, const float* lam,
                            float rate, float* state, const int* seq_starts, const int* slots, void* y, int y_dtype,
-                           int B, int W, int bw, int longest, hipStream_t stream) {
+                           int B, int T, int W, int bw, int longest, hipStream_t stream) {
     HB_REQUIRE(B > 0 && W > 0 && B <= 65535, "recurrent unit: empty input or too many sequences for the grid");
     HB_REQUIRE(bw > 0 && W % bw == 0, "recurrent unit: %d channels in blocks of %d", W, bw);
     if (longest >= LRU_RUNS_FROM) {
+        const size_t total = (size_t)T * W;
+        HB_REQUIRE(T > 0 && (total + 255) / 256 <= 0x7fffffffu, "recurrent unit: %d tokens of %d channels exceed the grid", T, W);
+        lru_decay_input_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(ug, gates, rb, ib, lam, rate, W, bw, total);
+        HB_CHECK_LAUNCH("lru_decay_input");
         const dim3 grid(B, (W + 63) / 64);
         if (y_dtype == HB_F32)
-            lru_scan_runs_kernel<float, LRU_RUNS><<<grid, 64 * LRU_RUNS, 0, stream>>>(ug, gates, rb, ib, lam, rate, state, seq_starts, slots, (float*)y, W, bw);
+            lru_scan_runs_kernel<float, LRU_RUNS><<<grid, 64 * LRU_RUNS, 0, stream>>>(ug, gates, state, seq_starts, slots, (float*)y, W, bw);
         else if (y_dtype == HB_BF16)
-            lru_scan_runs_kernel<bf16, LRU_RUNS><<<grid, 64 * LRU_RUNS, 0, stream>>>(ug, gates, rb, ib, lam, rate, state, seq_starts, slots, (bf16*)y, W, bw);
+            lru_scan_runs_kernel<bf16, LRU_RUNS><<<grid, 64 * LRU_RUNS, 0, stream>>>(ug, gates, state, seq_starts, slots, (bf16*)y, W, bw);
         else
             HB_REQUIRE(false, "recurrent unit: unknown output dtype %d", y_dtype);
         HB_CHECK_LAUNCH("lru_scan_runs");

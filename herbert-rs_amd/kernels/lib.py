@@ -46,7 +46,7 @@ SIGNATURES = {
         "hb_gated_delta": [_P, _I, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
         "hb_filter_state": [_P, _I, _P, _P, _P, _I, _I, _I, _P, _P],
         "hb_lru_inputs": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
-        "hb_lru_scan": [_P, _P, _P, _P, _P, _F, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+        "hb_lru_scan": [_P, _P, _P, _P, _P, _F, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
         "hb_gated_head_norm": [_P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _P],
         "hb_channel_decay": [_P, _I, _P, _P, _P, _I, _I, _I, _P],
     },

@@ -163,8 +163,9 @@ def lru_scan(ug, gates, r_bias, i_bias, lam, rate, state, meta, out, block):
     i = sigmoid(i_pre + i_bias), a = exp(-rate r softplus(lam)): S <- a S + sqrt(1 - a^2) i u, out = S g, where
     ug f32 [T, 2 W] = [u | g] and gates f32 [T, 2 W] holds, for every block of `block` channels, that block's
     r_pre then its i_pre; state f32 [slots, W] advanced in place; out [T, W] in any dtype. Where a sequence brings
-    128 tokens or more (meta.max_new) the walk is cut into runs that are walked side by side and joined, which
-    differs from the one walk by float32 rounding."""
+    128 tokens or more (meta.max_new) a kernel first turns `gates` into decays and inputs where they lie (gates is
+    overwritten), and the walk is cut into runs that are walked side by side and joined, which differs from the one
+    walk by float32 rounding."""
     T, W2 = ug.shape
     W = W2 // 2
     _check(ug, "ug", torch.float32, (T, 2 * W))
@@ -177,4 +178,4 @@ def lru_scan(ug, gates, r_bias, i_bias, lam, rate, state, meta, out, block):
     _check(meta.slots, "slots", torch.int32, (meta.num_seqs,))
     lib.call("recurrent", "hb_lru_scan", ug.data_ptr(), gates.data_ptr(), r_bias.data_ptr(), i_bias.data_ptr(),
              lam.data_ptr(), float(rate), state.data_ptr(), meta.seq_starts.data_ptr(), meta.slots.data_ptr(),
-             out.data_ptr(), dtype_code(out), meta.num_seqs, W, int(block), int(meta.max_new), _stream())
+             out.data_ptr(), dtype_code(out), meta.num_seqs, T, W, int(block), int(meta.max_new), _stream())
