@@ -826,8 +826,10 @@ extern "C" int hb_normed_pair(const float* a, const float* wa, float ca, const f
 //     are kept at size hd >= max(dim, vdim), the entries beyond a head's own size are zeros.
 // TK: the taps' count where it is 2, 3 or 4 (the filter's loop is then unrolled and all of a thread's loads of an
 // iteration are in flight together), 0: any count.
-template <class TQ, class TC, int TK>
-__global__ void __launch_bounds__(256)
+// NT: threads a token: a quarter of 1024 where the step has many tokens, 1024 where it has few (a token's
+// channels are then spread over sixteen waves, which hide each other's waits).
+template <class TQ, class TC, int TK, int NT>
+__global__ void __launch_bounds__(NT)
 filter_norm_rotate_write_kernel(const float* __restrict__ proj, int ld, const float* __restrict__ taps, int K,
                                 float* __restrict__ filter_state, const float* __restrict__ q_norm_w,
                                 const float* __restrict__ k_norm_w, const double* __restrict__ rates, int rot_dims,
@@ -836,6 +838,7 @@ filter_norm_rotate_write_kernel(const float* __restrict__ proj, int ld, const fl
                                 const int* __restrict__ page_table, int max_pages, int page_size,
                                 TQ* __restrict__ q_out, TC* __restrict__ k_cache, TC* __restrict__ v_cache, int nq,
                                 int nkv, int dim, int vdim, int hd, float eps, int moves_state) {
+    constexpr int U = NT == 256 ? 8 : 4;          // channels a thread handles at a time
     extern __shared__ float filtered[];           // [C] the token's channels, then [rot_dims] cosines and sines
     __shared__ float red[16];
     const int t = blockIdx.x, tid = threadIdx.x;
@@ -849,64 +852,9 @@ filter_norm_rotate_write_kernel(const float* __restrict__ proj, int ld, const fl
     float* state = filter_state + (size_t)slot * (K > 1 ? K - 1 : 1) * C;
     const int page = page_table[(size_t)slot * max_pages + pos / page_size];       // (asked for early: used last)
     const int in_page = pos % page_size;
-    float sq = 0.f, sk = 0.f;
-    // eight channels a thread at a time, so that a tap's eight loads are in flight together (one channel after
-    // the other, every load would wait for the one before: the taps' count is not known when this is compiled)
-    for (int c0 = tid; c0 < C; c0 += 8 * 256) {
-        float y[8], wn[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            // the norm's weight of the channel, loaded here beside the filter's operands: the loops that store the
-            // heads then read LDS only and wait for no memory
-            const int c = c0 + u * 256;
-            y[u] = 0.f;
-            wn[u] = 1.f;
-            if (c < QD) { if (q_norm_w) wn[u] = q_norm_w[c]; }
-            else if (c < QD + KD) { if (k_norm_w) wn[u] = k_norm_w[c - QD]; }
-        }
-        if (taps == nullptr) {
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int c = c0 + u * 256;
-                if (c < C) y[u] = proj[(size_t)t * ld + c];
-            }
-        } else {
-            const int taps_n = TK > 0 ? TK : K;
-#pragma unroll
-            for (int j = 0; j < taps_n; ++j) {
-                const int s = at - (taps_n - 1) + j;
-                const float* row = s >= 0 ? proj + (size_t)(first + s) * ld : state + (size_t)(taps_n - 1 + s) * C;
-                float v[8], w[8];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    const int c = c0 + u * 256;
-                    v[u] = c < C ? row[c] : 0.f;
-                    w[u] = c < C ? taps[(size_t)c * taps_n + j] : 0.f;
-                }
-#pragma unroll
-                for (int u = 0; u < 8; ++u) y[u] = fmaf(w[u], v[u], y[u]);
-                // one token a sequence: this thread is the only reader of its channels' kept inputs and moves
-                // them on itself (each takes the place of the one before it, the last the token's own input)
-                if (moves_state && j > 0) {
-#pragma unroll
-                    for (int u = 0; u < 8; ++u) {
-                        const int c = c0 + u * 256;
-                        if (c < C) state[(size_t)(j - 1) * C + c] = v[u];
-                    }
-                }
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int c = c0 + u * 256;
-            if (c >= C) continue;
-            filtered[c] = y[u] * wn[u];
-            if (c < QD) sq = fmaf(y[u], y[u], sq);
-            else if (c < QD + KD) sk = fmaf(y[u], y[u], sk);
-        }
-    }
+    // (the angles first: their loads then wait beside the filter's, not after them)
     if (rates != nullptr) {
-        for (int i = tid; i < rot_dims / 2; i += 256) {
+        for (int i = tid; i < rot_dims / 2; i += NT) {
             // the angle and its reduction to [-pi, pi] in float64 (a few operations), sine and cosine of the reduced
             // angle in float32: a float64 sincos costs as much as the rest of the kernel
             const double a = (double)pos * rates[i];
@@ -916,6 +864,91 @@ filter_norm_rotate_write_kernel(const float* __restrict__ proj, int ld, const fl
             sincosf((float)r, &s, &c);
             cs[2 * i] = c;
             cs[2 * i + 1] = s;
+        }
+    }
+    float sq = 0.f, sk = 0.f;
+    // U channels a thread at a time, so that a tap's U loads are in flight together (one channel after
+    // the other, every load would wait for the one before: the taps' count is not known when this is compiled)
+    for (int c0 = tid; c0 < C; c0 += U * NT) {
+        float y[U], wn[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            // the norm's weight of the channel, loaded here beside the filter's operands: the loops that store the
+            // heads then read LDS only and wait for no memory
+            const int c = c0 + u * NT;
+            y[u] = 0.f;
+            wn[u] = 1.f;
+            if (c < QD) { if (q_norm_w) wn[u] = q_norm_w[c]; }
+            else if (c < QD + KD) { if (k_norm_w) wn[u] = k_norm_w[c - QD]; }
+        }
+        if (taps == nullptr) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int c = c0 + u * NT;
+                if (c < C) y[u] = proj[(size_t)t * ld + c];
+            }
+        } else {
+            if (TK > 0) {
+                // the taps' count is known: every load of the eight channels is asked for before anything is stored
+                // (a store into the state would hold back the loads behind it, which may read the state)
+                constexpr int N = TK > 0 ? TK : 1;
+                float v[N][U], w[N][U];
+#pragma unroll
+                for (int j = 0; j < N; ++j) {
+                    const int s = at - (N - 1) + j;
+                    const float* row = s >= 0 ? proj + (size_t)(first + s) * ld : state + (size_t)(N - 1 + s) * C;
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        const int c = c0 + u * NT;
+                        v[j][u] = c < C ? row[c] : 0.f;
+                        w[j][u] = c < C ? taps[(size_t)c * N + j] : 0.f;
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < N; ++j)
+#pragma unroll
+                    for (int u = 0; u < U; ++u) y[u] = fmaf(w[j][u], v[j][u], y[u]);
+                // one token a sequence: this thread is the only reader of its channels' kept inputs and moves
+                // them on itself (each takes the place of the one before it, the last the token's own input)
+                if (moves_state) {
+#pragma unroll
+                    for (int j = 1; j < N; ++j)
+#pragma unroll
+                        for (int u = 0; u < U; ++u) {
+                            const int c = c0 + u * NT;
+                            if (c < C) state[(size_t)(j - 1) * C + c] = v[j][u];
+                        }
+                }
+            } else {
+                for (int j = 0; j < K; ++j) {
+                    const int s = at - (K - 1) + j;
+                    const float* row = s >= 0 ? proj + (size_t)(first + s) * ld : state + (size_t)(K - 1 + s) * C;
+                    float v[U], w[U];
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        const int c = c0 + u * NT;
+                        v[u] = c < C ? row[c] : 0.f;
+                        w[u] = c < C ? taps[(size_t)c * K + j] : 0.f;
+                    }
+#pragma unroll
+                    for (int u = 0; u < U; ++u) y[u] = fmaf(w[u], v[u], y[u]);
+                    if (moves_state && j > 0) {
+#pragma unroll
+                        for (int u = 0; u < U; ++u) {
+                            const int c = c0 + u * NT;
+                            if (c < C) state[(size_t)(j - 1) * C + c] = v[u];
+                        }
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int c = c0 + u * NT;
+            if (c >= C) continue;
+            filtered[c] = y[u] * wn[u];
+            if (c < QD) sq = fmaf(y[u], y[u], sq);
+            else if (c < QD + KD) sk = fmaf(y[u], y[u], sk);
         }
     }
     sq = hb_block_sum(sq, red);           // (its barriers also publish `filtered` and the angles)
@@ -933,11 +966,11 @@ filter_norm_rotate_write_kernel(const float* __restrict__ proj, int ld, const fl
         const float co = cs[2 * i], si = cs[2 * i + 1];
         return (d & 1) ? v * co + u * si : u * co - v * si;
     };
-    for (int idx = tid; idx < nq * hd; idx += 256) {
+    for (int idx = tid; idx < nq * hd; idx += NT) {
         const int h = idx / hd, d = idx - h * hd;
         q_out[(size_t)t * nq * hd + idx] = hb_from_float<TQ>(turned(h * dim, d, inv_q));
     }
-    for (int idx = tid; idx < nkv * hd; idx += 256) {
+    for (int idx = tid; idx < nkv * hd; idx += NT) {
         const int g = idx / hd, d = idx - g * hd;
         const size_t base = ((size_t)page * nkv + g) * page_size * hd;
         k_cache[base + (size_t)in_page * hd + d] = hb_from_float<TC>(turned(QD + g * dim, d, inv_k));
@@ -967,11 +1000,16 @@ extern "C" int hb_filter_norm_rotate_write(const float* proj, int ld, const floa
     // longest: the most tokens that a sequence of the step brings; at one the kernel moves the filter's state on
     // itself, otherwise hb_filter_state does so afterwards
     const int moves_state = longest == 1 && K > 1;
-#define HB_FNRW(TQ, TC, TK)                                                                                              \
-    filter_norm_rotate_write_kernel<TQ, TC, TK><<<T, 256, lds, stream>>>(                                                  \
+#define HB_FNRW_NT(TQ, TC, TK, NT)                                                                                       \
+    filter_norm_rotate_write_kernel<TQ, TC, TK, NT><<<T, NT, lds, stream>>>(                                              \
         proj, ld, taps, K, filter_state, q_norm_w, k_norm_w, rates, rot_dims, positions, seq_of, seq_starts, slots,       \
         page_table, max_pages, page_size, (TQ*)q_out, (TC*)k_cache, (TC*)v_cache, nq, nkv, dim, vdim, hd, eps,   \
         moves_state)
+#define HB_FNRW(TQ, TC, TK)                                                                                              \
+    do {                                                                                                                 \
+        if (T <= 64) HB_FNRW_NT(TQ, TC, TK, 1024);                                                                       \
+        else HB_FNRW_NT(TQ, TC, TK, 256);                                                                                \
+    } while (0)
 #define HB_FNRW_TAPS(TQ, TC)                                                                                             \
     do {                                                                                                                 \
         if (K == 4) HB_FNRW(TQ, TC, 4);                                                                                  \
@@ -987,6 +1025,7 @@ extern "C" int hb_filter_norm_rotate_write(const float* proj, int ld, const floa
         HB_REQUIRE(false, "filtered attention: unknown dtype %d", dtype);
 #undef HB_FNRW_TAPS
 #undef HB_FNRW
+#undef HB_FNRW_NT
     HB_CHECK_LAUNCH("filter_norm_rotate_write");
     return 0;
 }
