@@ -237,7 +237,9 @@ def test_prepared_attention_with_a_sink_and_a_far_key(nq, nkv, dim, vdim, K, rot
         part = RotaryPairs(rot["base"], rot_dims, None if sc is None else (sc["factor"], sc["low"], sc["high"], sc["original"]))
         rates = torch.tensor(part.pair_rates_host(), dtype=torch.float64, device=DEV)
     g = lambda t: None if t is None else t.to(DEV).contiguous()
-    for again in range(2):               # the second pass finds the slots, pages and filter rows used
+    # three passes: the later ones find the slots, pages and filter rows used, and ask the matrix cores' prompt kernels
+    # for their tiles of 64 and of 32 tokens by name (the first pass leaves the choice to the host)
+    for again, height in enumerate((None, 64, 32)):
         a, b = cache.alloc_slot(), cache.alloc_slot()
         got, got_short, got_q = [], [], []
         steps = [(2, 2), (61, 3), (2, 1), (85, 3)] + [(1, 0)] * (L - 150)
@@ -252,7 +254,7 @@ def test_prepared_attention_with_a_sink_and_a_far_key(nq, nkv, dim, vdim, K, rot
             ops.filter_norm_rotate_write(p, g(taps), state, g(qw), g(kw), rates, rot_dims, meta, kv, q, nq, nkv, dim, vdim, hd, eps)
             attn = torch.full_like(q, 9.0)
             if dtype == torch.bfloat16 and mfma.attention_supported(q, kv, nq, nkv, hd):
-                mfma.attention(q, meta, kv, attn, nq, nkv, hd, scale, 0, sinks=g(sinks))
+                mfma.attention(q, meta, kv, attn, nq, nkv, hd, scale, 0, sinks=g(sinks), tile_height=height if meta.max_new > 1 else None)
             else:
                 ops.attention_plain(q, meta, kv, attn, nq, nkv, hd, scale, 0, sinks=g(sinks))
             gated = torch.empty(T, nq * vdim, dtype=dtype, device=DEV)
