@@ -798,9 +798,61 @@ __global__ void normed_pair_kernel(const float* __restrict__ a, const float* __r
     }
 }
 
+// The same for rows of up to 4096 numbers in steps of four: both rows stay in registers between the two passes.
+template <bool ACCUM>
+__global__ void __launch_bounds__(256)
+normed_pair_held_kernel(const float* __restrict__ a, const float* __restrict__ wa, float ca,
+                        const float* __restrict__ b, const float* __restrict__ wb, float cb, float* out, int H, float eps) {
+    __shared__ float red[16];
+    const size_t row = (size_t)blockIdx.x * H;
+    const int quads = H / 4;
+    float4 ha[4], hb[4];
+    float sa = 0.f, sb = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int q = threadIdx.x + j * 256;
+        if (q < quads) {
+            ha[j] = *(const float4*)(a + row + 4 * q);
+            hb[j] = *(const float4*)(b + row + 4 * q);
+            sa += ha[j].x * ha[j].x + ha[j].y * ha[j].y + ha[j].z * ha[j].z + ha[j].w * ha[j].w;
+            sb += hb[j].x * hb[j].x + hb[j].y * hb[j].y + hb[j].z * hb[j].z + hb[j].w * hb[j].w;
+        }
+    }
+    sa = hb_block_sum(sa, red);
+    sb = hb_block_sum(sb, red);
+    const float ia = ca / sqrtf(sa / (float)H + eps), ib = cb / sqrtf(sb / (float)H + eps);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int q = threadIdx.x + j * 256;
+        if (q < quads) {
+            const float4 ga = *(const float4*)(wa + 4 * q), gb = *(const float4*)(wb + 4 * q);
+            float4 v;
+            v.x = ha[j].x * ia * ga.x + hb[j].x * ib * gb.x;
+            v.y = ha[j].y * ia * ga.y + hb[j].y * ib * gb.y;
+            v.z = ha[j].z * ia * ga.z + hb[j].z * ib * gb.z;
+            v.w = ha[j].w * ia * ga.w + hb[j].w * ib * gb.w;
+            float4* o = (float4*)(out + row + 4 * q);
+            if (ACCUM) {
+                const float4 p = *o;
+                v.x += p.x, v.y += p.y, v.z += p.z, v.w += p.w;
+            }
+            *o = v;
+        }
+    }
+}
+
 extern "C" int hb_normed_pair(const float* a, const float* wa, float ca, const float* b, const float* wb, float cb,
                               float* out, int R, int H, float eps, int accumulate, hipStream_t stream) {
     HB_REQUIRE(R > 0 && H > 0, "normed pair: empty input (R=%d, H=%d)", R, H);
+    if (H % 4 == 0 && H >= 1024 && H <= 4096 &&
+        (((uintptr_t)a | (uintptr_t)b | (uintptr_t)wa | (uintptr_t)wb | (uintptr_t)out) & 15) == 0) {
+        if (accumulate)
+            normed_pair_held_kernel<true><<<R, 256, 0, stream>>>(a, wa, ca, b, wb, cb, out, H, eps);
+        else
+            normed_pair_held_kernel<false><<<R, 256, 0, stream>>>(a, wa, ca, b, wb, cb, out, H, eps);
+        HB_CHECK_LAUNCH("normed_pair_held");
+        return 0;
+    }
     const int threads = H >= 1024 ? 256 : H >= 256 ? 128 : 64;
     if (accumulate)
         normed_pair_kernel<true><<<R, threads, 0, stream>>>(a, wa, ca, b, wb, cb, out, H, eps);

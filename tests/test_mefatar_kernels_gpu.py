@@ -41,7 +41,7 @@ def test_scaled_sum_then_norm(H):
     assert torch.allclose(xg.cpu(), want_x, atol=1e-6, rtol=1e-6)
 
 
-@pytest.mark.parametrize("H", [24, 72, 1536])
+@pytest.mark.parametrize("H", [24, 72, 1536, 2052, 4096])
 def test_two_normed_outputs_joined(H):
     a, b = rand(6, H, seed=1, scale=5.0), rand(6, H, seed=2, scale=0.2)            # of very different sizes
     wa, wb = 1 + 0.2 * rand(H, seed=3), 0.7 + 0.2 * rand(H, seed=4)
