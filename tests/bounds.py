@@ -31,7 +31,9 @@ F32_ABS = 1e-4
 #  it goes from 9e-6 for one layer to 1.1e-5 for 36)
 # ("vip": the Vipalorn configurations, whose recurrence, scores and routing stay float32; "mod": the Modasun
 #  configurations, the same and a float32 stream that is normed after every sum; "mef": the Mefatar
-#  configurations, whose stream, scores, recurrences and gates stay float32.)
+#  configurations, whose stream, scores, recurrences and gates stay float32: worst seen 0.04 to 0.08 for most, 0.10
+#  to 0.11 on single rows of the narrowest (widths of 64 and 72 through seven to nine layer runs, vocabularies of
+#  96 to 320), which is why its model-level tests let one row in fifty pass the bound by half.)
 BF16_REL_L2 = {"mef": 0.03, "mod": 0.03, "vip": 0.03, "A": 0.012, "B": 0.018, "C": 0.018, "D": 0.02, "F": 0.02, "wide": 0.02, "odd": 0.02, "random": 0.02, "long": 0.025, "deep": 0.02}
 BF16_REL_RMS = {"mef": 0.1, "mod": 0.1, "vip": 0.1, "A": 0.04, "B": 0.05, "C": 0.05, "D": 0.05, "F": 0.05, "wide": 0.08, "odd": 0.04, "random": 0.06, "long": 0.08, "deep": 0.08}
 
