@@ -6,6 +6,7 @@ from .qwen3 import Qwen3Config
 from .vipalorn import VipalornConfig
 from .modasun import ModasunConfig
 from .mefatar import MefatarConfig
+from .bozasun import BozasunConfig
 
-__all__ = ["Architecture", "ChatFormat", "MefatarConfig", "ModasunConfig", "Qwen3Config", "VipalornConfig", "load_config", "read_config_json",
+__all__ = ["Architecture", "BozasunConfig", "ChatFormat", "MefatarConfig", "ModasunConfig", "Qwen3Config", "VipalornConfig", "load_config", "read_config_json",
            "register_architecture", "registered_architectures", "resolve_architecture"]

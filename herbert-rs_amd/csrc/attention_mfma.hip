@@ -48,6 +48,28 @@ __device__ __forceinline__ int perm(int rho) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// The first key that a query at `pos` sees: with chunk > 0 the first position of its chunk of `chunk`
+// positions (counted from the sequence's start), else with window > 0 the first of the last `window`
+// positions, else 0. It never falls as pos grows.
+__device__ __forceinline__ int first_visible(int pos, int window, int chunk) {
+    if (chunk > 0) return pos / chunk * chunk;
+    return (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+}
+
+// Capped scores: s <- cap tanh(s / cap), in the units of the raw dot products (cap = softcap / scale, so that
+// the scaled score is softcap tanh(scale s / softcap)). tanh t = 1 - 2 / (1 + e^(2t)): e^(2t) infinite gives 1,
+// zero gives -1.
+__device__ __forceinline__ void cap_scores(f32x16 st[2], float cap) {
+    const float k = 2.0f * 1.4426950408889634f / cap;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const float e = fast_exp2(st[kb][i] * k);
+            st[kb][i] = cap - 2.0f * cap * __builtin_amdgcn_rcpf(1.0f + e);
+        }
+}
+
 // accumulator element i of lane group g2 of key block kb -> key within the page
 __device__ __forceinline__ int acc_key(int kb, int g2, int i) { return kb * 32 + 16 * (i >> 3) + 8 * g2 + (i & 7); }
 
@@ -277,7 +299,8 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache
                     const int* __restrict__ tile_seq, const int* __restrict__ tile_row0,
                     const int* __restrict__ tile_rows, const int* __restrict__ positions,
                     const int* __restrict__ slots, const int* __restrict__ page_table, int max_pages, int nq,
-                    int nkv, float c, int window, int per_tile, const float* __restrict__ sinks) {
+                    int nkv, float c, int window, int per_tile, const float* __restrict__ sinks, int chunked,
+                    float cap) {
     constexpr int KCH = HD / 8;                   // 16-byte chunks of a key row
     constexpr int KRPB = 128 / HD > 0 ? 128 / HD : 1;   // key rows in 256 bytes
     constexpr int KROWS = 512 / HD;               // key rows a load instruction brings (1 KB)
@@ -312,9 +335,10 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache
     const int pos0 = positions[row0];
     const int my_row = c32 < rows ? c32 : rows - 1;
     const int pos_q = pos0 + my_row;
-    const int lo_q = (window > 0 && pos_q + 1 > window) ? pos_q + 1 - window : 0;
+    const int lo_q = first_visible(pos_q, window, chunked);
     const int hi_tile = pos0 + rows - 1;                                     // last visible key
-    const int lo_tile = (window > 0 && pos0 + 1 > window) ? pos0 + 1 - window : 0;
+    const int lo_tile = first_visible(pos0, window, chunked);
+    const int lo_last = first_visible(hi_tile, window, chunked);            // what the tile's last query sees first
     const int first_page = lo_tile / PAGE, last_page = hi_tile / PAGE;
     // this group's pages: first_page + grp, + 2, ...; the first group has as many as the second or one more
     const int steps = (last_page - first_page) / 2 + 1;                      // of the first group: every wave loops so often
@@ -397,7 +421,8 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache
         float corr, mc;
         // a page that every query of the tile sees whole needs no mask
         const int page0 = page_of(i) * PAGE;
-        if (page0 + PAGE - 1 <= pos0 && (window == 0 || page0 >= hi_tile + 1 - window))
+        if (cap != 0.f) cap_scores(st, cap);
+        if (page0 + PAGE - 1 <= pos0 && page0 >= lo_last)
             mc = softmax_reference<false>(st, g2, page0, lo_q, pos_q, c, m, corr);
         else
             mc = softmax_reference<true>(st, g2, page0, lo_q, pos_q, c, m, corr);
@@ -476,7 +501,7 @@ attn_prefill_long_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
                          const int* __restrict__ tile_rows, const int* __restrict__ positions,
                          const int* __restrict__ slots, const int* __restrict__ page_table, int max_pages,
                          int nq, int nkv, float c, int window, int per_tile,
-                         const float* __restrict__ sinks) {
+                         const float* __restrict__ sinks, int chunked, float cap) {
     constexpr int KCH = HD / 8;
     constexpr int KRPB = 128 / HD > 0 ? 128 / HD : 1;
     constexpr int KROWS = 512 / HD;
@@ -510,10 +535,11 @@ attn_prefill_long_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
     const int pos0 = tile_pos0 + (rows > 0 ? 32 * half : 0);
     const int my_row = rows > 0 ? (c32 < rows ? c32 : rows - 1) : 0;
     const int pos_q = pos0 + my_row;
-    const int lo_q = (window > 0 && pos_q + 1 > window) ? pos_q + 1 - window : 0;
+    const int lo_q = first_visible(pos_q, window, chunked);
     const int hi_half = pos0 + (rows > 0 ? rows : 1) - 1;                     // last key this half sees
+    const int lo_last = first_visible(hi_half, window, chunked);             // what the half's last query sees first
     // the workgroup's pages: from the first a row of the tile sees to the last
-    const int lo_tile = (window > 0 && tile_pos0 + 1 > window) ? tile_pos0 + 1 - window : 0;
+    const int lo_tile = first_visible(tile_pos0, window, chunked);
     const int first_page = lo_tile / PAGE, last_page = (tile_pos0 + tile_n - 1) / PAGE;
     const int steps = last_page - first_page + 1;
     const int mine = active ? hi_half / PAGE - first_page + 1 : 0;            // this half's steps: pages up to its own last
@@ -587,7 +613,8 @@ attn_prefill_long_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
         if (i >= mine) return;
         float corr, mc;
         const int page0 = page_of(i) * PAGE;
-        if (page0 + PAGE - 1 <= pos0 && (window == 0 || page0 >= hi_half + 1 - window))
+        if (cap != 0.f) cap_scores(st, cap);
+        if (page0 + PAGE - 1 <= pos0 && page0 >= lo_last)
             mc = softmax_reference<false>(st, g2, page0, lo_q, pos_q, c, m, corr);
         else
             mc = softmax_reference<true>(st, g2, page0, lo_q, pos_q, c, m, corr);
@@ -664,7 +691,8 @@ attn_decode_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_cache, bf16*
                    const int* __restrict__ context_lens, const int* __restrict__ slots,
                    const int* __restrict__ page_table, int max_pages, int nq, int nkv, float c, int window,
                    int pages_per_split, DecodeFusion fu, bf16* __restrict__ out,
-                   const int* __restrict__ ranges, int n_seqs, const float* __restrict__ sinks) {
+                   const int* __restrict__ ranges, int n_seqs, const float* __restrict__ sinks, int chunked,
+                   float cap) {
     // ranges == null: the grid is (sequence, kv head, range), every sequence cut into gridDim.z
     // ranges of pages_per_split pages (those past a sequence's end hold nothing).
     // ranges != null (sequences of unequal lengths): the grid is (1, kv head, item);
@@ -690,7 +718,7 @@ attn_decode_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_cache, bf16*
     const int G = nq / nkv;
     const int ctx = context_lens[b];                 // keys 0 .. ctx-1; the query sits at ctx-1
     const int hi = ctx - 1;
-    const int lo = (window > 0 && ctx > window) ? ctx - window : 0;
+    const int lo = first_visible(hi, window, chunked);
     const int first_page = lo / PAGE + split * pages_per_split;
     int last_page = first_page + pages_per_split - 1;
     if (last_page > hi / PAGE) last_page = hi / PAGE;
@@ -883,6 +911,7 @@ attn_decode_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_cache, bf16*
         if (page_idx < last_page) LOAD_K(page_idx + 1)
         float corr;
         bf16x8 pb[2][2];
+        if (cap != 0.f) cap_scores(st, cap);
         if (page_idx * PAGE >= lo && page_idx * PAGE + PAGE - 1 <= hi)
             softmax_page<false>(st, g2, page_idx * PAGE, lo, hi, c, m, l, corr, pb);
         else
@@ -1017,10 +1046,11 @@ extern "C" int hb_attn_prefill_mfma(const void* q, const void* k_cache, const vo
                                     int num_tiles, const int* positions, const int* slots,
                                     const int* page_table, int max_pages, int page_size, int nq, int nkv,
                                     int hd, float scale, int window, int tile_height, const float* sinks,
-                                    hipStream_t stream) {
+                                    int chunk, float softcap, hipStream_t stream) {
     HB_REQUIRE(num_tiles > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attn_prefill: bad sizes");
     HB_REQUIRE(page_size == PAGE, "attn_prefill: pages must hold %d tokens", PAGE);
-    HB_REQUIRE(window >= 0, "attn_prefill: bad window");
+    HB_REQUIRE(window >= 0 && chunk >= 0 && !(window > 0 && chunk > 0), "attn_prefill: bad window or chunk");
+    HB_REQUIRE(softcap >= 0.f, "attn_prefill: the scores' cap must be positive (0: none)");
     HB_REQUIRE(scale > 0.f, "attn_prefill: the score scale must be positive");
     HB_REQUIRE(tile_height == 32 || tile_height == 64, "attn_prefill: tiles are 32 or 64 tokens high");
     const int G = nq / nkv;
@@ -1028,6 +1058,7 @@ extern "C" int hb_attn_prefill_mfma(const void* q, const void* k_cache, const vo
     HB_REQUIRE((long)num_tiles * per_tile < (1l << 30), "attn_prefill: too many tiles");
     const int total = num_tiles * per_tile;
     const float c = scale * LOG2E;
+    const float cap = softcap / scale;          // in the units of the raw dot products
     // tiles of 32 tokens: two groups of waves, each with two stages of keys and two of values;
     // tiles of 64: one ring of three stages of keys and three of values
     const size_t lds = (size_t)(tile_height == 64 ? 6 : 8) * PAGE * hd * sizeof(bf16);
@@ -1042,7 +1073,8 @@ extern "C" int hb_attn_prefill_mfma(const void* q, const void* k_cache, const vo
         }                                                                                                \
         KERNEL<HDV><<<total, 512, lds, stream>>>((const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache, \
                                                  (bf16*)out, tile_seq, tile_row0, tile_rows, positions, slots, \
-                                                 page_table, max_pages, nq, nkv, c, window, per_tile, sinks); \
+                                                 page_table, max_pages, nq, nkv, c, window, per_tile, sinks, \
+                                                 chunk, cap); \
     } while (0)
     if (tile_height == 64) {
         if (hd == 32) LAUNCH_PREFILL(attn_prefill_long_kernel, 32);
@@ -1069,11 +1101,13 @@ extern "C" int hb_attn_decode_mfma(const void* q, void* k_cache, void* v_cache, 
                                    int pages_per_split, const float* qkv, const float* q_norm_w,
                                    const float* k_norm_w, const float* cos_t, const float* sin_t, float eps,
                                    int write_kv, int qkv_slices, size_t slice_stride, const int* ranges,
-                                   float q_temp_coef, int q_temp_every, const float* sinks, hipStream_t stream) {
+                                   float q_temp_coef, int q_temp_every, const float* sinks, int chunk,
+                                   float softcap, hipStream_t stream) {
     // ranges != null: see attn_decode_kernel; `splits` is then the number of items of the grid (the
     // partial results are [nq, splits]), pages_per_split is not read
-    HB_REQUIRE(!ranges || (B >= 2 && splits >= 2 && window == 0),
+    HB_REQUIRE(!ranges || (B >= 2 && splits >= 2 && window == 0 && chunk == 0),
                "attn_decode: a list of ranges is for two sequences or more, with a merge, without a window");
+    HB_REQUIRE(chunk >= 0 && !(window > 0 && chunk > 0) && softcap >= 0.f, "attn_decode: bad chunk or cap");
     HB_REQUIRE(B > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attn_decode: bad sizes");
     HB_REQUIRE(page_size == PAGE, "attn_decode: pages must hold %d tokens", PAGE);
     HB_REQUIRE(nq / nkv <= 32, "attn_decode: more than 32 query heads share a kv head");
@@ -1091,7 +1125,7 @@ extern "C" int hb_attn_decode_mfma(const void* q, void* k_cache, void* v_cache, 
     HB_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "attn_decode: cos and sin tables come together");
 #define DECODE_ARGS(QPTR) QPTR, (bf16*)k_cache, (bf16*)v_cache, partial_o, partial_ml, context_lens, slots, \
                           page_table, max_pages, nq, nkv, c, window, pages_per_split, fu, direct, ranges, B, \
-                          direct ? sinks : nullptr
+                          direct ? sinks : nullptr, chunk, softcap / scale
 #define LAUNCH_DECODE(HDV) do {                                                                          \
     if (qkv)                                                                                             \
         attn_decode_kernel<HDV, true><<<grid, 64, 0, stream>>>(DECODE_ARGS(nullptr));                    \

@@ -12,6 +12,9 @@
 // all float32. The window is not in the reference, which never reads those keys. Nor is the sink: with
 // `sinks` [nq] given, the softmax's denominator of head h also holds exp(sinks[h]), a score without a key
 // and a value, unscaled, counted once (the running maximum starts there and the running sum at one).
+// Nor are these two: with chunk > 0 the keys a query sees are those at or before it within its own chunk of
+// `chunk` positions, [floor(p / chunk) chunk, p], the chunks counted from the sequence's start; with
+// softcap > 0 a scaled score s becomes softcap tanh(s / softcap) before the softmax.
 #include "common.h"
 #include <math.h>
 
@@ -27,7 +30,7 @@ attention_plain_kernel(const TQ* __restrict__ q, const TC* __restrict__ k_cache,
                        const int* __restrict__ positions, const int* __restrict__ seq_of,
                        const int* __restrict__ slots, const int* __restrict__ page_table, int max_pages,
                        int page_size, int nq, int nkv, int hd, float scale, int window,
-                       const float* __restrict__ sinks) {
+                       const float* __restrict__ sinks, int chunk, float softcap) {
     __shared__ float qs[HB_MAX_HEAD_DIM];
     __shared__ float ps[HB_WAVE];
     const int t = blockIdx.x;
@@ -43,7 +46,7 @@ attention_plain_kernel(const TQ* __restrict__ q, const TC* __restrict__ k_cache,
     __syncthreads();
 
     const int hi = pos + 1;
-    const int lo = (window > 0 && hi > window) ? hi - window : 0;
+    const int lo = chunk > 0 ? pos / chunk * chunk : (window > 0 && hi > window) ? hi - window : 0;
     float m = -INFINITY, l = 0.f;
     if (sinks) m = sinks[h], l = 1.0f;
     float acc[ACC_REGS];
@@ -60,6 +63,7 @@ attention_plain_kernel(const TQ* __restrict__ q, const TC* __restrict__ k_cache,
             float dot = 0.f;
             for (int d = 0; d < hd; ++d) dot = fmaf(qs[d], hb_to_float(kr[d]), dot);
             s = dot * scale;
+            if (softcap > 0.f) s = softcap * tanhf(s / softcap);
         }
         const float m_new = fmaxf(m, hb_wave_max(s));
         const float corr = expf(m - m_new);
@@ -102,22 +106,23 @@ extern "C" int hb_attention_plain(const void* q, const void* k_cache, const void
                                   int dtype, const int* positions, const int* seq_of, const int* slots,
                                   const int* page_table, int max_pages, int page_size, int T, int nq,
                                   int nkv, int hd, float scale, int window, const float* sinks,
-                                  hipStream_t stream) {
+                                  int chunk, float softcap, hipStream_t stream) {
     HB_REQUIRE(T > 0 && nq > 0 && nkv > 0, "attention: empty input");
     HB_REQUIRE(nq % nkv == 0, "attention: %d query heads not divisible by %d kv heads", nq, nkv);
     HB_REQUIRE(hd > 0 && hd <= HB_MAX_HEAD_DIM, "attention: head_dim %d not in 1..%d", hd,
                HB_MAX_HEAD_DIM);
     HB_REQUIRE(page_size > 0 && window >= 0, "attention: bad page size or window");
+    HB_REQUIRE(chunk >= 0 && !(chunk > 0 && window > 0) && softcap >= 0.f, "attention: bad chunk or cap of the scores");
     HB_REQUIRE(nq <= 65535, "attention: too many heads for the grid");
     dim3 grid(T, nq);
     if (dtype == HB_F32)
         attention_plain_kernel<float, float, float><<<grid, HB_WAVE, 0, stream>>>(
             (const float*)q, (const float*)k_cache, (const float*)v_cache, (float*)out, positions, seq_of,
-            slots, page_table, max_pages, page_size, nq, nkv, hd, scale, window, sinks);
+            slots, page_table, max_pages, page_size, nq, nkv, hd, scale, window, sinks, chunk, softcap);
     else if (dtype == HB_BF16)
         attention_plain_kernel<bf16, bf16, bf16><<<grid, HB_WAVE, 0, stream>>>(
             (const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, positions, seq_of,
-            slots, page_table, max_pages, page_size, nq, nkv, hd, scale, window, sinks);
+            slots, page_table, max_pages, page_size, nq, nkv, hd, scale, window, sinks, chunk, softcap);
     else
         HB_REQUIRE(false, "attention: unknown dtype %d", dtype);
     HB_CHECK_LAUNCH("attention_plain");

@@ -870,8 +870,11 @@ extern "C" int hb_normed_pair(const float* a, const float* wa, float ca, const f
 //     before the step's first row from the slot's state [K - 1, C] (zeros in a fresh slot); the state is
 //     moved on by a kernel of its own afterwards (hb_filter_state in the module of the recurrent mixers), or
 //     here where every sequence brings one token;
+//   bias (null: none): bias[c] is added to channel c after the filter;
 //   norm (weights null: none): all queries of the token are divided by their common root mean square and
-//     multiplied by q_norm_w [nq x dim], the keys likewise with k_norm_w [nkv x dim];
+//     multiplied by q_norm_w [nq x dim], the keys likewise with k_norm_w [nkv x dim]; with head_norm every
+//     query head and every key head is divided by its own root mean square instead, and the weights are
+//     q_norm_w [dim] and k_norm_w [dim], the same for every head;
 //   rotation (rates null: none): entries 2i and 2i + 1 of the first rot_dims of every query and key head turn
 //     by position x rates[i]; rates and the angle are float64, sine and cosine float32 of the angle reduced to [-pi, pi];
 //   q_out [T, nq x hd], key pages [page, kv head, token, hd], value pages [page, kv head, hd, token]: heads
@@ -889,9 +892,10 @@ filter_norm_rotate_write_kernel(const float* __restrict__ proj, int ld, const fl
                                 const int* __restrict__ seq_starts, const int* __restrict__ slots,
                                 const int* __restrict__ page_table, int max_pages, int page_size,
                                 TQ* __restrict__ q_out, TC* __restrict__ k_cache, TC* __restrict__ v_cache, int nq,
-                                int nkv, int dim, int vdim, int hd, float eps, int moves_state) {
+                                int nkv, int dim, int vdim, int hd, float eps, int moves_state,
+                                const float* __restrict__ bias, int head_norm) {
     constexpr int U = NT == 256 ? 8 : 4;          // channels a thread handles at a time
-    extern __shared__ float filtered[];           // [C] the token's channels, then [rot_dims] cosines and sines
+    extern __shared__ float filtered[];           // [C] the token's channels, then [rot_dims] cosines and sines, then [nq + nkv] a head's 1 / rms
     __shared__ float red[16];
     const int t = blockIdx.x, tid = threadIdx.x;
     const int QD = nq * dim, KD = nkv * dim, C = QD + KD + nkv * vdim;
@@ -928,8 +932,9 @@ filter_norm_rotate_write_kernel(const float* __restrict__ proj, int ld, const fl
             // the norm's weight of the channel, loaded here beside the filter's operands: the loops that store the
             // heads then read LDS only and wait for no memory
             const int c = c0 + u * NT;
-            y[u] = 0.f;
+            y[u] = (bias != nullptr && c < C) ? bias[c] : 0.f;
             wn[u] = 1.f;
+            if (head_norm) continue;                  // (a head's weights are applied where the heads are stored)
             if (c < QD) { if (q_norm_w) wn[u] = q_norm_w[c]; }
             else if (c < QD + KD) { if (k_norm_w) wn[u] = k_norm_w[c - QD]; }
         }
@@ -937,7 +942,7 @@ filter_norm_rotate_write_kernel(const float* __restrict__ proj, int ld, const fl
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const int c = c0 + u * NT;
-                if (c < C) y[u] = proj[(size_t)t * ld + c];
+                if (c < C) y[u] += proj[(size_t)t * ld + c];
             }
         } else {
             if (TK > 0) {
@@ -1008,10 +1013,25 @@ filter_norm_rotate_write_kernel(const float* __restrict__ proj, int ld, const fl
     const float inv_q = q_norm_w ? 1.0f / sqrtf(sq / (float)QD + eps) : 1.0f;
     const float inv_k = k_norm_w ? 1.0f / sqrtf(sk / (float)KD + eps) : 1.0f;
     const int rd = rates != nullptr ? rot_dims : 0;
+    float* const inv_head = cs + rd;
+    if (head_norm) {
+        // a wave a head: its sum of squares in one order whatever else the step holds
+        const int lane = tid & 63;
+        for (int h = tid >> 6; h < nq + nkv; h += NT / 64) {
+            float ss = 0.f;
+            for (int d = lane; d < dim; d += 64) ss = fmaf(filtered[h * dim + d], filtered[h * dim + d], ss);
+            ss = hb_wave_sum(ss);
+            if (lane == 0) inv_head[h] = 1.0f / sqrtf(ss / (float)dim + eps);
+        }
+        __syncthreads();
+    }
     // one entry of a query or key head after norm and rotation; c0: the head's first channel
     auto turned = [&](int c0, int d, float inv) {
         if (d >= dim) return 0.f;
-        auto normed = [&](int e) { return filtered[c0 + e] * inv; };        // (the weight is in `filtered` already)
+        const float* const hw = !head_norm ? nullptr : c0 < QD ? q_norm_w : k_norm_w;
+        if (head_norm) inv = inv_head[c0 / dim];
+        // (without head_norm the weight is in `filtered` already)
+        auto normed = [&](int e) { return filtered[c0 + e] * inv * (hw ? hw[e] : 1.0f); };
         if (d >= rd) return normed(d);
         const int i = d >> 1;
         const float u = normed(2 * i), v = normed(2 * i + 1);
@@ -1037,7 +1057,7 @@ extern "C" int hb_filter_norm_rotate_write(const float* proj, int ld, const floa
                                            const int* seq_starts, const int* slots, const int* page_table,
                                            int max_pages, int page_size, void* q_out, void* k_cache, void* v_cache,
                                            int dtype, int T, int nq, int nkv, int dim, int vdim, int hd, float eps,
-                                           int longest, hipStream_t stream) {
+                                           int longest, const float* bias, int head_norm, hipStream_t stream) {
     HB_REQUIRE(T > 0 && nq > 0 && nkv > 0 && dim > 0 && vdim > 0, "filtered attention: empty input");
     HB_REQUIRE(hd >= dim && hd >= vdim, "filtered attention: heads kept at %d cannot hold %d and %d", hd, dim, vdim);
     const long long C = (long long)(nq + nkv) * dim + (long long)nkv * vdim;
@@ -1046,7 +1066,8 @@ extern "C" int hb_filter_norm_rotate_write(const float* proj, int ld, const floa
     HB_REQUIRE(taps == nullptr || K == 1 || filter_state != nullptr, "filtered attention: a filter needs its state");
     HB_REQUIRE(rates == nullptr || (rot_dims > 0 && rot_dims % 2 == 0 && rot_dims <= dim),
                "filtered attention: %d rotated entries of heads of %d", rot_dims, dim);
-    const size_t lds = ((size_t)C + (rates ? rot_dims : 0)) * sizeof(float);
+    HB_REQUIRE(!head_norm || (q_norm_w != nullptr && k_norm_w != nullptr), "filtered attention: a norm a head needs its weights");
+    const size_t lds = ((size_t)C + (rates ? rot_dims : 0) + (head_norm ? nq + nkv : 0)) * sizeof(float);
     HB_REQUIRE(lds <= 60 * 1024, "filtered attention: %lld channels a token do not fit the kernel's LDS", C);
     if (taps == nullptr) K = 0;
     // longest: the most tokens that a sequence of the step brings; at one the kernel moves the filter's state on
@@ -1056,7 +1077,7 @@ extern "C" int hb_filter_norm_rotate_write(const float* proj, int ld, const floa
     filter_norm_rotate_write_kernel<TQ, TC, TK, NT><<<T, NT, lds, stream>>>(                                              \
         proj, ld, taps, K, filter_state, q_norm_w, k_norm_w, rates, rot_dims, positions, seq_of, seq_starts, slots,       \
         page_table, max_pages, page_size, (TQ*)q_out, (TC*)k_cache, (TC*)v_cache, nq, nkv, dim, vdim, hd, eps,   \
-        moves_state)
+        moves_state, bias, head_norm)
 #define HB_FNRW(TQ, TC, TK)                                                                                              \
     do {                                                                                                                 \
         if (T <= 64) HB_FNRW_NT(TQ, TC, TK, 1024);                                                                       \
@@ -1079,6 +1100,21 @@ extern "C" int hb_filter_norm_rotate_write(const float* proj, int ld, const floa
 #undef HB_FNRW
 #undef HB_FNRW_NT
     HB_CHECK_LAUNCH("filter_norm_rotate_write");
+    return 0;
+}
+
+// ------------------------------------------- a bias a column
+// x[t, c] += bias[c]: the bias of a projection whose product adds to these rows.
+__global__ void add_bias_kernel(float* __restrict__ x, const float* __restrict__ bias, int H, size_t total) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx < total) x[idx] += bias[idx % H];
+}
+
+extern "C" int hb_add_bias(float* x, const float* bias, int T, int H, hipStream_t stream) {
+    HB_REQUIRE(T > 0 && H > 0, "bias: empty input");
+    const size_t total = (size_t)T * H;
+    add_bias_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(x, bias, H, total);
+    HB_CHECK_LAUNCH("add_bias");
     return 0;
 }
 
@@ -1112,5 +1148,103 @@ extern "C" int hb_gate_heads(const void* attn, int dtype, const float* gate_rows
     else
         HB_REQUIRE(false, "gate: unknown dtype %d", dtype);
     HB_CHECK_LAUNCH("gate_heads");
+    return 0;
+}
+
+// ------------------------------------------- a token's own input to the residual stream, layer by layer
+// With e = table[token, col0 .. col0 + D) (a token's row of a table, this layer's part of it):
+//     g = gelu_tanh(W_gate x) * e;   y = W_proj g;   x <- x + y / sqrt(mean(y^2) + eps) * w
+// x f32 [T, H] in place; W_gate [D, H], W_proj [H, D] and the table in one storage type; all arithmetic float32.
+// A workgroup takes TPB tokens: their rows of x lie in LDS, a wave takes gate rows in turn (a row of W_gate is
+// read once for all TPB tokens, the lanes share its columns), then a thread takes output columns (a row of
+// W_proj each), and the rows' sums of squares are added up by the block in a fixed order.
+template <class TW, int TPB>
+__global__ void __launch_bounds__(256)
+token_side_kernel(float* __restrict__ x, const int* __restrict__ tokens, const TW* __restrict__ table, int table_ld,
+                  int col0, const TW* __restrict__ w_gate, const TW* __restrict__ w_proj,
+                  const float* __restrict__ norm_w, int T, int H, int D, float eps) {
+    extern __shared__ float side_lds[];            // [TPB][H] rows of x, then of y; [TPB][D] g
+    __shared__ float red[16];
+    float* const xs = side_lds;
+    float* const gs = side_lds + (size_t)TPB * H;
+    const int t0 = blockIdx.x * TPB, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int nt = T - t0 < TPB ? T - t0 : TPB;
+    for (int i = tid; i < TPB * H; i += 256) {
+        const int k = i / H;
+        xs[i] = k < nt ? x[(size_t)(t0 + k) * H + (i - k * H)] : 0.f;
+    }
+    __syncthreads();
+    for (int j = wave; j < D; j += 4) {
+        float acc[TPB];
+#pragma unroll
+        for (int k = 0; k < TPB; ++k) acc[k] = 0.f;
+        for (int c = lane; c < H; c += 64) {
+            const float w = hb_to_float(w_gate[(size_t)j * H + c]);
+#pragma unroll
+            for (int k = 0; k < TPB; ++k) acc[k] = fmaf(w, xs[k * H + c], acc[k]);
+        }
+#pragma unroll
+        for (int k = 0; k < TPB; ++k) {
+            const float z = hb_wave_sum(acc[k]);
+            if (lane == 0 && k < nt) {
+                const float gelu = 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+                gs[k * D + j] = gelu * hb_to_float(table[(size_t)tokens[t0 + k] * table_ld + col0 + j]);
+            }
+        }
+    }
+    __syncthreads();
+    float ss[TPB];
+#pragma unroll
+    for (int k = 0; k < TPB; ++k) ss[k] = 0.f;
+    for (int c = tid; c < H; c += 256) {
+        float y[TPB];
+#pragma unroll
+        for (int k = 0; k < TPB; ++k) y[k] = 0.f;
+        for (int j = 0; j < D; ++j) {
+            const float w = hb_to_float(w_proj[(size_t)c * D + j]);
+#pragma unroll
+            for (int k = 0; k < TPB; ++k) y[k] = fmaf(w, gs[k * D + j], y[k]);
+        }
+#pragma unroll
+        for (int k = 0; k < TPB; ++k) {
+            xs[k * H + c] = y[k];                      // (this thread alone reads and writes column c from here on)
+            ss[k] = fmaf(y[k], y[k], ss[k]);
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < TPB; ++k) ss[k] = hb_block_sum(ss[k], red);
+    for (int c = tid; c < H; c += 256) {
+        const float w = norm_w[c];
+#pragma unroll
+        for (int k = 0; k < TPB; ++k)
+            if (k < nt) x[(size_t)(t0 + k) * H + c] += xs[k * H + c] / sqrtf(ss[k] / (float)H + eps) * w;
+    }
+}
+
+extern "C" int hb_token_side(float* x, const int* tokens, const void* table, int table_ld, int col0, const void* w_gate,
+                             const void* w_proj, int dtype, const float* norm_w, int T, int H, int D, float eps,
+                             hipStream_t stream) {
+    HB_REQUIRE(T > 0 && H > 0 && D > 0, "token input: empty input");
+    HB_REQUIRE(col0 >= 0 && col0 + D <= table_ld, "token input: the layer's columns lie outside the table's rows");
+    const size_t per_token = ((size_t)H + D) * sizeof(float);
+    HB_REQUIRE(per_token <= 60 * 1024, "token input: a row of %d and %d gates do not fit the kernel's LDS", H, D);
+    const bool four = 4 * per_token <= 60 * 1024 && T >= 4;
+    const size_t lds = (four ? 4 : 1) * per_token;
+#define HB_SIDE(TW)                                                                                                   \
+    do {                                                                                                              \
+        if (four)                                                                                                     \
+            token_side_kernel<TW, 4><<<(T + 3) / 4, 256, lds, stream>>>(x, tokens, (const TW*)table, table_ld, col0,   \
+                                                                        (const TW*)w_gate, (const TW*)w_proj, norm_w, \
+                                                                        T, H, D, eps);                                \
+        else                                                                                                          \
+            token_side_kernel<TW, 1><<<T, 256, lds, stream>>>(x, tokens, (const TW*)table, table_ld, col0,            \
+                                                              (const TW*)w_gate, (const TW*)w_proj, norm_w, T, H, D,  \
+                                                              eps);                                                   \
+    } while (0)
+    if (dtype == HB_F32) HB_SIDE(float);
+    else if (dtype == HB_BF16) HB_SIDE(bf16);
+    else HB_REQUIRE(false, "token input: unknown dtype %d", dtype);
+#undef HB_SIDE
+    HB_CHECK_LAUNCH("token_side");
     return 0;
 }

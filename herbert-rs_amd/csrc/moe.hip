@@ -71,19 +71,31 @@ moe_route_kernel(const float* __restrict__ logits, int ld, const float* __restri
 // the experts form n_groups equal runs of adjacent experts, a group is worth the two highest of its
 // selection values, added; only the experts of the `keep` best groups can be chosen (the lower index of equals,
 // for groups as for experts), and the chosen experts' scores are divided by their sum + 1e-20.
+// Three parameters change the form: softmax_scores (s is the softmax of the logits over all E experts instead of
+// their sigmoids), worth_top (how many of a group's highest selection values make its worth: 2, or 1), renorm
+// (0: the weights are the chosen experts' scores as they are).
 // One wave a token; the scores lie in LDS.
 __global__ void __launch_bounds__(HB_WAVE)
 moe_route_scores_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ correction,
                         int* __restrict__ chosen, float* __restrict__ weight, int E, int top, int n_groups,
-                        int keep) {
+                        int keep, int softmax_scores, int worth_top, int renorm) {
     __shared__ float score[HB_WAVE * MOE_MAX_E_PER_LANE];
     __shared__ float choice[HB_WAVE * MOE_MAX_E_PER_LANE];
     __shared__ float worth[HB_WAVE * MOE_MAX_E_PER_LANE];
     __shared__ int kept[HB_WAVE * MOE_MAX_E_PER_LANE];
     const int t = blockIdx.x, lane = threadIdx.x;
     const int size = E / n_groups;
+    float top_logit = -INFINITY, denom = 1.0f;
+    if (softmax_scores) {
+        for (int e = lane; e < E; e += HB_WAVE) top_logit = fmaxf(top_logit, logits[(size_t)t * ld + e]);
+        top_logit = hb_wave_max(top_logit);
+        float part = 0.f;
+        for (int e = lane; e < E; e += HB_WAVE) part += expf(logits[(size_t)t * ld + e] - top_logit);
+        denom = hb_wave_sum(part);
+    }
     for (int e = lane; e < E; e += HB_WAVE) {
-        const float s = 1.0f / (1.0f + expf(-logits[(size_t)t * ld + e]));
+        const float z = logits[(size_t)t * ld + e];
+        const float s = softmax_scores ? expf(z - top_logit) / denom : 1.0f / (1.0f + expf(-z));
         score[e] = s;
         choice[e] = s + (correction ? correction[e] : 0.f);
     }
@@ -99,7 +111,7 @@ moe_route_scores_kernel(const float* __restrict__ logits, int ld, const float* _
                 b = c;
             }
         }
-        worth[g] = size > 1 ? a + b : a;
+        worth[g] = (size > 1 && worth_top > 1) ? a + b : a;
     }
     __syncthreads();
     for (int g = lane; g < n_groups; g += HB_WAVE) {
@@ -147,6 +159,7 @@ moe_route_scores_kernel(const float* __restrict__ logits, int ld, const float* _
         for (int i = 0; i < MOE_MAX_E_PER_LANE; ++i)
             if (lane + HB_WAVE * i == at) z[i] = -INFINITY;
     }
+    if (!renorm) return;
     const float total = sum + 1e-20f;
     for (int j = lane; j < top; j += HB_WAVE) weight[(size_t)t * top + j] /= total;
 }
@@ -155,11 +168,12 @@ moe_route_scores_kernel(const float* __restrict__ logits, int ld, const float* _
 // Block e < E: the pairs of expert e, in the order of the pairs, to rows [first, first + count) and
 // the expert's tiles into the list; block E: the list's unused end. order[row] = pair,
 // row_of[pair] = row. Every block counts all experts' pairs for itself (a histogram in LDS), so that
-// no kernel has to run before it.
+// no kernel has to run before it. Experts from `real` on have no matrices (their output is their input): their
+// pairs get rows like any others, but their tiles are marked as holding nothing, so no product runs on them.
 __global__ void __launch_bounds__(256)
 moe_place_kernel(const int* __restrict__ chosen, int* __restrict__ counts, int* __restrict__ order,
                  int* __restrict__ row_of, int* __restrict__ tile_expert, int* __restrict__ tile_row0,
-                 int* __restrict__ tile_rows, int A, int E, int max_tiles) {
+                 int* __restrict__ tile_rows, int A, int E, int max_tiles, int real) {
     __shared__ int hist[HB_WAVE * MOE_MAX_E_PER_LANE];
     __shared__ int wave_n[4];
     __shared__ int base;
@@ -180,7 +194,7 @@ moe_place_kernel(const int* __restrict__ chosen, int* __restrict__ counts, int* 
     const int count = hist[e];
     if (threadIdx.x == 0) counts[e] = count;
     for (int i = threadIdx.x; i * MOE_TILE_M < count; i += blockDim.x) {
-        tile_expert[tile0 + i] = e;
+        tile_expert[tile0 + i] = e < real ? e : -1;
         tile_row0[tile0 + i] = first + i * MOE_TILE_M;
         tile_rows[tile0 + i] = count - i * MOE_TILE_M < MOE_TILE_M ? count - i * MOE_TILE_M : MOE_TILE_M;
     }
@@ -212,23 +226,25 @@ moe_place_kernel(const int* __restrict__ chosen, int* __restrict__ counts, int* 
 // by_scores 1: sigmoid scores, `bias` is the correction of the choice, n_groups groups of which `keep` count.
 extern "C" int hb_moe_route(const float* logits, const float* bias, int* chosen, float* weight, int* counts,
                             int* order, int* row_of, int* tile_expert, int* tile_row0, int* tile_rows, int T, int E,
-                            int top, int max_tiles, int ld, int by_scores, int n_groups, int keep,
-                            hipStream_t stream) {
+                            int top, int max_tiles, int ld, int by_scores, int n_groups, int keep, int real,
+                            int softmax_scores, int worth_top, int renorm, hipStream_t stream) {
     HB_REQUIRE(ld >= E, "moe: logits rows %d apart for %d experts", ld, E);
     HB_REQUIRE(!by_scores || (n_groups > 0 && E % n_groups == 0 && keep > 0 && keep <= n_groups &&
                               top <= keep * (E / n_groups)),
                "moe: %d of %d groups of %d experts cannot give %d experts", keep, n_groups, E, top);
     HB_REQUIRE(T > 0 && E > 0 && top > 0 && top <= E, "moe: %d of %d experts for %d tokens", top, E, T);
+    HB_REQUIRE(real > 0 && real <= E, "moe: %d of %d experts have matrices", real, E);
     HB_REQUIRE(E <= HB_WAVE * MOE_MAX_E_PER_LANE, "moe: %d experts, the router takes up to %d", E, HB_WAVE * MOE_MAX_E_PER_LANE);
     const long long A = (long long)T * top;
     HB_REQUIRE(A < (1ll << 30), "moe: too many (token, expert) pairs");
     HB_REQUIRE(max_tiles >= (A + MOE_TILE_M - 1) / MOE_TILE_M + E, "moe: the tile list is too short");
     if (by_scores)
-        moe_route_scores_kernel<<<T, HB_WAVE, 0, stream>>>(logits, ld, bias, chosen, weight, E, top, n_groups, keep);
+        moe_route_scores_kernel<<<T, HB_WAVE, 0, stream>>>(logits, ld, bias, chosen, weight, E, top, n_groups, keep,
+                                                           softmax_scores, worth_top, renorm);
     else
         moe_route_kernel<<<T, HB_WAVE, 0, stream>>>(logits, ld, bias, chosen, weight, E, top);
     HB_CHECK_LAUNCH("moe_route");
-    moe_place_kernel<<<E + 1, 256, 0, stream>>>(chosen, counts, order, row_of, tile_expert, tile_row0, tile_rows, (int)A, E, max_tiles);
+    moe_place_kernel<<<E + 1, 256, 0, stream>>>(chosen, counts, order, row_of, tile_expert, tile_row0, tile_rows, (int)A, E, max_tiles, real);
     HB_CHECK_LAUNCH("moe_place");
     return 0;
 }
@@ -352,9 +368,13 @@ extern "C" int hb_moe_activate(const float* gu, void* act, int act_dtype, int ro
 // ------------------------------------------------------------------------ combine
 // x[t, :] += sum_j weight[t, j] * y[row_of[t * top + j], :]    (float32, j ascending)
 // shared [T, H] (or null): a part that every token takes, added times sigmoid(gate[t * gate_ld]).
+// input [T, H] (or null) with chosen [T, top] and real: a pair whose expert is `real` or beyond has no row in y;
+// its output is the token's own input row.
+template <class TIn>
 __global__ void moe_combine_kernel(const float* __restrict__ y, const float* __restrict__ weight,
                                    const int* __restrict__ row_of, float* __restrict__ x, int top, int H,
-                                   const float* __restrict__ shared, const float* __restrict__ gate, int gate_ld) {
+                                   const float* __restrict__ shared, const float* __restrict__ gate, int gate_ld,
+                                   const TIn* __restrict__ input, const int* __restrict__ chosen, int real) {
     const int t = blockIdx.x;
     const float open = shared ? 1.0f / (1.0f + expf(-gate[(size_t)t * gate_ld])) : 0.f;
     // (a token's rows and weights once, eight at a time, then whole rows)
@@ -366,12 +386,14 @@ __global__ void moe_combine_kernel(const float* __restrict__ y, const float* __r
             const bool in = j0 + j < top;
             rows[j] = y + (size_t)row_of[(size_t)t * top + (in ? j0 + j : 0)] * H;
             w[j] = in ? weight[(size_t)t * top + j0 + j] : 0.f;
+            if (input != nullptr && in && chosen[(size_t)t * top + j0 + j] >= real) rows[j] = nullptr;
         }
         for (int i = threadIdx.x; i < H; i += blockDim.x) {
             float s = 0.f;
 #pragma unroll
             for (int j = 0; j < 8; ++j)
-                if (j0 + j < top) s = fmaf(w[j], rows[j][i], s);
+                if (j0 + j < top)
+                    s = fmaf(w[j], rows[j] != nullptr ? rows[j][i] : hb_to_float(input[(size_t)t * H + i]), s);
             if (shared && j0 == 0) s = fmaf(open, shared[(size_t)t * H + i], s);
             x[(size_t)t * H + i] += s;
         }
@@ -379,10 +401,18 @@ __global__ void moe_combine_kernel(const float* __restrict__ y, const float* __r
 }
 
 extern "C" int hb_moe_combine(const float* y, const float* weight, const int* row_of, float* x, int T, int top, int H,
-                              const float* shared, const float* gate, int gate_ld, hipStream_t stream) {
+                              const float* shared, const float* gate, int gate_ld, const void* input,
+                              int input_dtype, const int* chosen, int real, hipStream_t stream) {
     HB_REQUIRE(shared == nullptr || (gate != nullptr && gate_ld > 0), "moe combine: a shared part needs its gate");
     HB_REQUIRE(T > 0 && top > 0 && H > 0, "moe combine: empty input");
-    moe_combine_kernel<<<T, H >= 1024 ? 256 : 64, 0, stream>>>(y, weight, row_of, x, top, H, shared, gate, gate_ld);
+    HB_REQUIRE(input == nullptr || chosen != nullptr, "moe combine: experts without matrices need the choices");
+    const int threads = H >= 1024 ? 256 : 64;
+    if (input != nullptr && input_dtype == HB_BF16)
+        moe_combine_kernel<bf16><<<T, threads, 0, stream>>>(y, weight, row_of, x, top, H, shared, gate, gate_ld,
+                                                            (const bf16*)input, chosen, real);
+    else
+        moe_combine_kernel<float><<<T, threads, 0, stream>>>(y, weight, row_of, x, top, H, shared, gate, gate_ld,
+                                                             (const float*)input, chosen, real);
     HB_CHECK_LAUNCH("moe_combine");
     return 0;
 }

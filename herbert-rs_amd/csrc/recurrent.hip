@@ -19,20 +19,21 @@ __device__ __forceinline__ float hb_silu(float z) { return z / (1.0f + expf(-z))
 //   [n_unit sections of unit_dim channels | plain sections of plain_dim channels]
 // y[t, c] = silu(sum_j taps[c, j] * in[t - (K - 1) + j, c]), the inputs before the step's first row
 // from the slot's state [K - 1, C] (zeros in a fresh slot). A unit section is then divided by
-// sqrt(sum of squares + unit_eps); sections below n_scaled are also multiplied by `scale`.
+// sqrt(sum of squares + unit_eps); sections below n_scaled are also multiplied by `scale`. With bias [C] the
+// sum starts at bias[c]. The last plain section may be shorter than plain_dim (it ends with the channels).
 // One wave a (token, section).
 __global__ void __launch_bounds__(HB_WAVE)
 conv_silu_kernel(const float* __restrict__ proj, int ld, const float* __restrict__ taps,
                  const float* __restrict__ conv_state, const int* __restrict__ seq_of,
                  const int* __restrict__ seq_starts, const int* __restrict__ slots, float* __restrict__ out,
                  int C, int K, int n_unit, int unit_dim, int n_scaled, float scale, float unit_eps,
-                 int plain_dim) {
+                 int plain_dim, const float* __restrict__ bias) {
     const int t = blockIdx.x;
     const int sec = blockIdx.y;
     const int lane = threadIdx.x;
     const bool unit = sec < n_unit;
     const int c0 = unit ? sec * unit_dim : n_unit * unit_dim + (sec - n_unit) * plain_dim;
-    const int len = unit ? unit_dim : plain_dim;
+    const int len = unit ? unit_dim : (plain_dim < C - c0 ? plain_dim : C - c0);
     const int seq = seq_of[t];
     const int first = seq_starts[seq];
     const int at = t - first;                     // the token's place among the step's tokens of its sequence
@@ -41,7 +42,7 @@ conv_silu_kernel(const float* __restrict__ proj, int ld, const float* __restrict
     float ss = 0.f;
     for (int d = lane; d < len; d += HB_WAVE) {
         const int c = c0 + d;
-        float acc = 0.f;
+        float acc = bias ? bias[c] : 0.f;
         for (int j = 0; j < K; ++j) {
             const int s = at - (K - 1) + j;
             const float v = s >= 0 ? proj[(size_t)(first + s) * ld + c] : state[(size_t)(K - 1 + s) * C + c];
@@ -80,14 +81,16 @@ __global__ void conv_state_kernel(const float* __restrict__ proj, int ld, float*
 extern "C" int hb_conv_silu(const float* proj, int ld, const float* taps, float* conv_state, const int* seq_of,
                             const int* seq_starts, const int* slots, float* out, int T, int B, int C, int K,
                             int n_unit, int unit_dim, int n_scaled, float scale, float unit_eps, int n_plain,
-                            int plain_dim, hipStream_t stream) {
+                            int plain_dim, const float* bias, hipStream_t stream) {
     HB_REQUIRE(T > 0 && B > 0 && C > 0, "conv: empty input");
     HB_REQUIRE(K >= 1 && K <= HB_MAX_TAPS, "conv: %d taps, the kernel takes 1 to %d", K, HB_MAX_TAPS);
-    HB_REQUIRE(n_unit * unit_dim + n_plain * plain_dim == C && ld >= C, "conv: the sections do not add up to %d channels", C);
+    HB_REQUIRE(n_unit * unit_dim + n_plain * plain_dim >= C && (n_plain == 0 ? n_unit * unit_dim == C
+               : n_unit * unit_dim + (n_plain - 1) * plain_dim < C) && ld >= C,
+               "conv: the sections do not add up to %d channels", C);
     HB_REQUIRE(n_unit + n_plain <= 65535 && B <= 65535, "conv: too many sections or sequences for the grid");
     conv_silu_kernel<<<dim3(T, n_unit + n_plain), HB_WAVE, 0, stream>>>(
         proj, ld, taps, conv_state, seq_of, seq_starts, slots, out, C, K, n_unit, unit_dim, n_scaled, scale,
-        unit_eps, plain_dim);
+        unit_eps, plain_dim, bias);
     HB_CHECK_LAUNCH("conv_silu");
     if (K > 1) {
         conv_state_kernel<<<dim3(B, (C + 255) / 256), 256, 0, stream>>>(proj, ld, conv_state, seq_starts, slots, C, K, nullptr);
@@ -645,5 +648,148 @@ extern "C" int hb_channel_decay(const float* z, int ld, const float* A_log, cons
     channel_decay_kernel<<<(unsigned)(blocks > 16384 ? 16384 : blocks), 256, 0, stream>>>(z, ld, A_log, dt_bias, g,
                                                                                            D, heads * D, n);
     HB_CHECK_LAUNCH("channel_decay");
+    return 0;
+}
+
+// ------------------------------------------------- state-space layer with one decay a head
+// A head h (on group h / (heads / groups) of B and C) keeps S [N, P], zero when its sequence starts, and for
+// every token, with dt = softplus(dt_pre[h] + dt_bias[h]) and a = exp(-exp(A_log[h]) dt):
+//     S <- a S + dt B x^T;   y = S^T C + D[h] x.
+// u f32 [T, ldu]: a row's columns are [x: heads x P | B: groups x N | C: groups x N] (what the convolution
+// left); dt_pre: column dt_off + h of proj's rows (f32, ld apart); state f32 [slots, heads, N, P]; y f32
+// [T, heads x P]. Everything is float32.
+// A workgroup is one wave on (16 columns of S, head, sequence): a column's N numbers lie over 4 lanes, lane j
+// holding rows j, j + 4, ... (NR of them), so the sum over N is NR products a lane and two exchanges, in one
+// order whatever the step holds. The tokens are a chain; their inputs come through LDS eight tokens at a time,
+// so that the chain waits for memory once in eight steps.
+#define SSM_COLS 16
+#define SSM_TOKENS 8
+template <int NR>
+__global__ void __launch_bounds__(HB_WAVE)
+ssm_scan_kernel(const float* __restrict__ u, int ldu, const float* __restrict__ proj, int ld, int dt_off,
+                const float* __restrict__ dt_bias, const float* __restrict__ A_log, const float* __restrict__ Dskip,
+                float* __restrict__ state, const int* __restrict__ seq_starts, const int* __restrict__ slots,
+                float* __restrict__ y, int heads, int groups, int N, int P) {
+    extern __shared__ float ssm_lds[];     // [SSM_TOKENS][B: N | C: N | x: SSM_COLS | dt, a]
+    const int tile = blockIdx.x, h = blockIdx.y, seq = blockIdx.z;
+    const int lane = threadIdx.x, col = lane >> 2, part = lane & 3;
+    const int p = tile * SSM_COLS + col;
+    const bool live = p < P;
+    const int g = h / (heads / groups);
+    const int first = seq_starts[seq], n_tok = seq_starts[seq + 1] - first;
+    const int inner = heads * P;
+    const int stride = 2 * N + SSM_COLS + 2;
+    float* S = state + (((size_t)slots[seq] * heads + h) * N) * P;
+    float s[NR];
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+        const int n = part + 4 * i;
+        s[i] = (live && n < N) ? S[(size_t)n * P + p] : 0.f;
+    }
+    const float rate = expf(A_log[h]), bias = dt_bias[h], skip = Dskip[h];
+    for (int t0 = 0; t0 < n_tok; t0 += SSM_TOKENS) {
+        const int nt = n_tok - t0 < SSM_TOKENS ? n_tok - t0 : SSM_TOKENS;
+        __syncthreads();
+        for (int idx = lane; idx < nt * stride; idx += HB_WAVE) {
+            const int k = idx / stride, e = idx - k * stride;
+            const size_t row = (size_t)(first + t0 + k);
+            float v;
+            if (e < 2 * N) {
+                v = u[row * ldu + inner + (e < N ? g * N + e : (groups + g) * N + (e - N))];
+            } else if (e < 2 * N + SSM_COLS) {
+                const int pc = tile * SSM_COLS + (e - 2 * N);
+                v = pc < P ? u[row * ldu + h * P + pc] : 0.f;
+            } else {
+                const float z = proj[row * ld + dt_off + h] + bias;
+                const float dt = z > 20.f ? z : log1pf(expf(z));
+                v = e == 2 * N + SSM_COLS ? dt : expf(-rate * dt);
+            }
+            ssm_lds[idx] = v;
+        }
+        __syncthreads();
+        for (int k = 0; k < nt; ++k) {
+            const float* in = ssm_lds + k * stride;
+            const float x = in[2 * N + col], dt = in[2 * N + SSM_COLS], a = in[2 * N + SSM_COLS + 1];
+            const float dx = dt * x;
+            float acc = 0.f;
+#pragma unroll
+            for (int i = 0; i < NR; ++i) {
+                const int n = part + 4 * i;
+                if (n < N) {
+                    s[i] = fmaf(a, s[i], dx * in[n]);
+                    acc = fmaf(s[i], in[N + n], acc);
+                }
+            }
+            acc += __shfl_xor(acc, 1, HB_WAVE);
+            acc += __shfl_xor(acc, 2, HB_WAVE);
+            if (live && part == 0) y[(size_t)(first + t0 + k) * inner + h * P + p] = fmaf(skip, x, acc);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+        const int n = part + 4 * i;
+        if (live && n < N) S[(size_t)n * P + p] = s[i];
+    }
+}
+
+extern "C" int hb_ssm_scan(const float* u, int ldu, const float* proj, int ld, int dt_off, const float* dt_bias,
+                           const float* A_log, const float* Dskip, float* state, const int* seq_starts,
+                           const int* slots, float* y, int B, int heads, int groups, int N, int P,
+                           hipStream_t stream) {
+    HB_REQUIRE(B > 0 && heads > 0 && groups > 0 && N > 0 && P > 0, "state-space walk: empty input");
+    HB_REQUIRE(heads % groups == 0, "state-space walk: %d heads in %d groups", heads, groups);
+    HB_REQUIRE(N <= 256, "state-space walk: a state of %d rows, the kernel takes up to 256", N);
+    HB_REQUIRE(ldu >= heads * P + 2 * groups * N && dt_off >= 0 && dt_off + heads <= ld,
+               "state-space walk: the columns lie outside their rows");
+    HB_REQUIRE(heads <= 65535 && B <= 65535, "state-space walk: too many heads or sequences for the grid");
+    const dim3 grid((P + SSM_COLS - 1) / SSM_COLS, heads, B);
+    const size_t lds = (size_t)SSM_TOKENS * (2 * N + SSM_COLS + 2) * sizeof(float);
+#define HB_SSM(NRV) ssm_scan_kernel<NRV><<<grid, HB_WAVE, lds, stream>>>(u, ldu, proj, ld, dt_off, dt_bias, A_log, Dskip, \
+                                                                         state, seq_starts, slots, y, heads, groups, N, P)
+    if (N <= 16) HB_SSM(4);
+    else if (N <= 32) HB_SSM(8);
+    else if (N <= 64) HB_SSM(16);
+    else if (N <= 128) HB_SSM(32);
+    else HB_SSM(64);
+#undef HB_SSM
+    HB_CHECK_LAUNCH("ssm_scan");
+    return 0;
+}
+
+// ------------------------------------------------- gate, then a norm in groups: what leaves the state-space walk
+// v = o silu(z); y = v / sqrt(mean over the group of v^2 + eps) * w: a row of `width` is cut into `parts` equal
+// groups, each normed by its own root mean square; w [width]; z: columns [z_off, + width) of proj's rows.
+// One wave a (token, group).
+template <class TOut>
+__global__ void __launch_bounds__(HB_WAVE)
+gated_group_norm_kernel(const float* __restrict__ o, const float* __restrict__ proj, int ld, int z_off,
+                        const float* __restrict__ w, TOut* __restrict__ y, int width, int parts, float eps) {
+    const int t = blockIdx.x, part = blockIdx.y, lane = threadIdx.x;
+    const int len = width / parts, c0 = part * len;
+    const float* in = o + (size_t)t * width + c0;
+    const float* gate = proj + (size_t)t * ld + z_off + c0;
+    float ss = 0.f;
+    for (int d = lane; d < len; d += HB_WAVE) {
+        const float v = in[d] * hb_silu(gate[d]);
+        ss = fmaf(v, v, ss);
+    }
+    ss = hb_wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)len + eps);
+    for (int d = lane; d < len; d += HB_WAVE)
+        y[(size_t)t * width + c0 + d] = hb_from_float<TOut>(in[d] * hb_silu(gate[d]) * inv * w[c0 + d]);
+}
+
+extern "C" int hb_gated_group_norm(const float* o, const float* proj, int ld, int z_off, const float* w, void* y,
+                                   int y_dtype, int T, int width, int parts, float eps, hipStream_t stream) {
+    HB_REQUIRE(T > 0 && width > 0 && parts > 0 && width % parts == 0 && parts <= 65535,
+               "gated norm in groups: %d columns in %d groups", width, parts);
+    HB_REQUIRE(z_off >= 0 && z_off + width <= ld, "gated norm in groups: the gate's columns lie outside the rows");
+    if (y_dtype == HB_F32)
+        gated_group_norm_kernel<float><<<dim3(T, parts), HB_WAVE, 0, stream>>>(o, proj, ld, z_off, w, (float*)y, width, parts, eps);
+    else if (y_dtype == HB_BF16)
+        gated_group_norm_kernel<bf16><<<dim3(T, parts), HB_WAVE, 0, stream>>>(o, proj, ld, z_off, w, (bf16*)y, width, parts, eps);
+    else
+        HB_REQUIRE(false, "gated norm in groups: unknown output dtype %d", y_dtype);
+    HB_CHECK_LAUNCH("gated_group_norm");
     return 0;
 }

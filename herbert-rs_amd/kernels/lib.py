@@ -28,7 +28,9 @@ SIGNATURES = {
         "hb_rmsnorm_scaled_sum": [_P, _P, _P, _P, _P, _I, _I, _I, _F, _P],
         "hb_normed_pair": [_P, _P, _F, _P, _P, _F, _P, _I, _I, _F, _I, _P],
         "hb_filter_norm_rotate_write": [_P, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P,
-                                        _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+                                        _I, _I, _I, _I, _I, _I, _I, _F, _I, _P, _I, _P],
+        "hb_add_bias": [_P, _P, _I, _I, _P],
+        "hb_token_side": [_P, _P, _P, _I, _I, _P, _P, _I, _P, _I, _I, _I, _F, _P],
         "hb_gate_heads": [_P, _I, _P, _I, _I, _P, _I, _I, _I, _I, _P],
         "hb_fill_u32": [_P, _U32, _SZ, _P],
         "hb_layernorm": [_P, _P, _F, _P, _P, _I, _P, _I, _I, _F, _P],
@@ -42,7 +44,9 @@ SIGNATURES = {
         "hb_gemm_plain_batched": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _SZ, _SZ, _SZ, _P],
     },
     "recurrent": {
-        "hb_conv_silu": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _I, _P],
+        "hb_conv_silu": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _I, _P, _P],
+        "hb_ssm_scan": [_P, _I, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+        "hb_gated_group_norm": [_P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _P],
         "hb_gated_delta": [_P, _I, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
         "hb_filter_state": [_P, _I, _P, _P, _P, _I, _I, _I, _P, _P],
         "hb_lru_inputs": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
@@ -56,14 +60,14 @@ SIGNATURES = {
         "hb_latent_attention_plain": [_P, _P, _P, _I, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
     },
     "moe": {
-        "hb_moe_route": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
+        "hb_moe_route": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P],
         "hb_moe_gemm_plain": [_P, _I, _P, _I, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _P],
         "hb_moe_activate": [_P, _P, _I, _I, _I, _F, _F, _F, _P],
-        "hb_moe_combine": [_P, _P, _P, _P, _I, _I, _I, _P, _P, _I, _P],
+        "hb_moe_combine": [_P, _P, _P, _P, _I, _I, _I, _P, _P, _I, _P, _I, _P, _I, _P],
         "hb_grouped_mfma": [_P, _I, _SZ, _P, _I, _I, _P, _I, _SZ, _I, _P, _I, _P, _P, _P, _I, _I, _I, _F, _F, _F, _I, _P],
     },
     "attention_plain": {
-        "hb_attention_plain": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P],
+        "hb_attention_plain": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _I, _F, _P],
     },
     "sampling": {
         "hb_argmax": [_P, _I, _I, _I, _P, _P, _P, _I, _P],

@@ -387,9 +387,9 @@ def gemm_swiglu(a, w_interleaved, out, packed=False, norm=None, tile=0, row_scal
 
 
 lib.register_signatures("attention_mfma", {
-    "hb_attn_prefill_mfma": [_P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P],
+    "hb_attn_prefill_mfma": [_P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P, _I, _F, _P],
     "hb_attn_decode_mfma": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I,
-                            _P, _P, _P, _P, _P, _F, _I, _I, ctypes.c_size_t, _P, _F, _I, _P, _P],
+                            _P, _P, _P, _P, _P, _F, _I, _I, ctypes.c_size_t, _P, _F, _I, _P, _I, _F, _P],
 })
 
 ATTENTION_HEAD_DIMS = (32, 64, 128)
@@ -454,15 +454,15 @@ def _prefill_tiles(meta, height=QUERY_TILE):
 DECODE_WAVES = 1024       # waves of the decode kernel that the 256 CUs hold at a time
 
 
-def _decode_split(meta, nkv, window):
+def _decode_split(meta, nkv, window, chunk=0):
     """(ranges, pages per range): as many ranges as still give no more waves than the GPU holds at
     a time, every range at least one page. With one range the kernel writes the output itself and
     no merge runs. (Measured at 4 K tokens a sequence: what costs is a second, partly filled round
     of waves. 48 sequences x 8 kv heads: 2 ranges, 768 waves, 9.8 ms a step; 3 ranges, 1152 waves,
     10.6 ms. 40 sequences: 3 ranges, 960 waves, 8.9 ms; 4 ranges, 1280 waves, 10.0 ms.)"""
     span = (meta.context_bucket + 63) // 64     # by bucket, so that a captured graph's grid stays right
-    if window:
-        span = min(span, (window + 63) // 64 + 1)
+    if window or chunk:
+        span = min(span, ((window or chunk) + 63) // 64 + 1)     # a chunk's keys lie on as many pages as a window's
     pairs = meta.num_seqs * nkv
     if 2 * pairs >= DECODE_WAVES:
         # (how evenly the waves sit is a matter of the sequences themselves: padding rows' waves end at once)
@@ -491,7 +491,7 @@ def _decode_split(meta, nkv, window):
     return best
 
 
-def _decode_ranges(meta, nkv, window):
+def _decode_ranges(meta, nkv, window, chunk=0):
     """(items of the grid, list of ranges on the GPU) for a step whose contexts are of very unequal
     lengths, else None. Equal shares would leave the waves of the short sequences with nothing and
     those of the long ones with all the work (one sequence of 32 K tokens beside seven of 1 K: 128 of
@@ -500,7 +500,7 @@ def _decode_ranges(meta, nkv, window):
     fewer than two a sequence, and the lengths are unequal enough for more than one round of waves
     to pay). The list changes with every step and is read by the kernel; the grid does not change."""
     B = meta.num_seqs
-    if not meta.unequal or window or B < 2 or meta.max_new != 1:
+    if not meta.unequal or window or chunk or B < 2 or meta.max_new != 1:
         return None
     # at least two items a sequence, so that a range is no longer than the mean sequence: beyond
     # half a round of sequences the grid is more than one round of waves (the kernel's limit: 1,024 items)
@@ -583,15 +583,18 @@ def attention_decode_fused(qkv, q_norm_w, k_norm_w, cos, sin, meta, kv, out, nq,
              window, splits, per, src, None if q_norm_w is None else q_norm_w.data_ptr(),
              None if k_norm_w is None else k_norm_w.data_ptr(), None if cos is None else cos.data_ptr(),
              None if sin is None else sin.data_ptr(), float(eps), 1, n_slices, stride,
-             None if ranges is None else ranges.data_ptr(), coef, every, None, _stream())
+             None if ranges is None else ranges.data_ptr(), coef, every, None, 0, 0.0, _stream())
 
 
 DEFERRED_SLICES = (2, 4, 8)     # numbers of slices of the projection that the decode kernel adds up itself
 
 
-def attention(q, meta, kv, out, nq, nkv, hd, scale, window, tile_height=None, scratch=None, sinks=None):
+def attention(q, meta, kv, out, nq, nkv, hd, scale, window, tile_height=None, scratch=None, sinks=None, chunk=None,
+              softcap=None):
     """Causal (and windowed) attention of the step's tokens over their slots' pages.
     sinks f32 [nq]: the softmax's denominator of head h also holds exp(sinks[h]), once, without key or value.
+    chunk: a query sees the keys of its own chunk of that many positions only, the chunks counted from the
+    sequence's start (not together with a window). softcap: a scaled score s becomes softcap tanh(s / softcap).
     One token a sequence: the split decode kernel; otherwise one of the two tiled prompt kernels
     (tile_height 32 or 64 asks for one by name; None: the host's choice, see _prefill_tile_height)."""
     T = q.shape[0]
@@ -604,7 +607,7 @@ def attention(q, meta, kv, out, nq, nkv, hd, scale, window, tile_height=None, sc
     _check(meta.slots, "slots", torch.int32, (meta.num_seqs,))
     if not attention_supported(q, kv, nq, nkv, hd):
         raise BackendError(f"attention_mfma refuses head_dim {hd} with {nq}/{nkv} heads")
-    window = int(window or 0)
+    window, chunk, softcap = int(window or 0), int(chunk or 0), float(softcap or 0.0)
     if sinks is not None:
         _check(sinks, "sinks", torch.float32, (nq,))
     sinks_ptr = None if sinks is None else sinks.data_ptr()
@@ -612,18 +615,18 @@ def attention(q, meta, kv, out, nq, nkv, hd, scale, window, tile_height=None, sc
         if T != meta.num_seqs:
             raise BackendError("decode attention needs one token for each sequence")
         _check(meta.context_lens, "context_lens", torch.int32, (T,))
-        listed = _decode_ranges(meta, nkv, window)
+        listed = _decode_ranges(meta, nkv, window, chunk)
         if listed:
             (splits, ranges), per = listed, 1
             po, pml = _partial_buffers(scratch, q.device, nq, splits, hd)
         else:
-            (splits, per), ranges = _decode_split(meta, nkv, window), None
+            (splits, per), ranges = _decode_split(meta, nkv, window, chunk), None
             po, pml = _partial_buffers(scratch, q.device, T * nq, splits, hd)
         lib.call("attention_mfma", "hb_attn_decode_mfma", q.data_ptr(), kv.k.data_ptr(), kv.v.data_ptr(),
                  out.data_ptr(), po.data_ptr(), pml.data_ptr(), meta.context_lens.data_ptr(),
                  meta.slots.data_ptr(), kv.page_table.data_ptr(), kv.page_table.shape[1], kv.page_size,
                  T, nq, nkv, hd, float(scale), window, splits, per, None, None, None, None, None, 0.0, 0, 1, 0,
-                 None if ranges is None else ranges.data_ptr(), 0.0, 0, sinks_ptr, _stream())
+                 None if ranges is None else ranges.data_ptr(), 0.0, 0, sinks_ptr, chunk, softcap, _stream())
         return
     _check(meta.positions, "positions", torch.int32, (T,))
     height = tile_height or _prefill_tile_height(meta, nkv, nq // nkv)
@@ -633,4 +636,5 @@ def attention(q, meta, kv, out, nq, nkv, hd, scale, window, tile_height=None, sc
     lib.call("attention_mfma", "hb_attn_prefill_mfma", q.data_ptr(), kv.k.data_ptr(), kv.v.data_ptr(),
              out.data_ptr(), tile_seq.data_ptr(), tile_row0.data_ptr(), tile_rows.data_ptr(), n_tiles,
              meta.positions.data_ptr(), meta.slots.data_ptr(), kv.page_table.data_ptr(),
-             kv.page_table.shape[1], kv.page_size, nq, nkv, hd, float(scale), window, height, sinks_ptr, _stream())
+             kv.page_table.shape[1], kv.page_size, nq, nkv, hd, float(scale), window, height, sinks_ptr, chunk, softcap,
+             _stream())

@@ -19,7 +19,9 @@ class Routing:
     """The buffers that routing fills for a step of T tokens: chosen int32 [T, top], weight f32 [T, top],
     order / row_of int32 [T top], the tiles' lists."""
 
-    def __init__(self, ints, weight, T, E, top):
+    def __init__(self, ints, weight, T, E, top, real=None):
+        """real: the first `real` of the E experts have matrices (None: all); the others' output is their input."""
+        self.real = E if real is None else int(real)
         A, tiles = T * top, max_tiles(T * top, E)
         need = 3 * A + E + 3 * tiles
         if ints.numel() < need or ints.dtype != torch.int32:
@@ -40,13 +42,19 @@ class Routing:
         return 3 * T * top + E + 3 * max_tiles(T * top, E)
 
 
-def route(logits, bias, routing, scores=False, groups=1, keep=1):
+def route(logits, bias, routing, scores=False, groups=1, keep=1, score="sigmoid", worth_top=2, renorm=True):
     """logits f32 [T, E] (+ bias f32 [E]) -> routing (see Routing): the largest logits + bias, weighed by a
     softmax over the chosen. The logits' rows may be wider than E (their first E columns count).
     scores=True: s = sigmoid(logit), the choice runs on s + bias within the `keep` best of `groups` equal
     runs of adjacent experts (a group is worth its top two selection values), and the weights are the chosen
-    experts' s over their sum."""
+    experts' s over their sum. score="softmax": s is the softmax of the logits over all experts; worth_top 1: a
+    group is worth its highest selection value alone; renorm False: the weights are the chosen experts' s as they are.
+    Experts from routing.real on have no matrices: their pairs' tiles are marked as holding nothing."""
     r = routing
+    if score not in ("sigmoid", "softmax") or worth_top not in (1, 2):
+        raise BackendError(f"routing: scores are 'sigmoid' or 'softmax', a group is worth its top 1 or 2, not {score!r}, {worth_top}")
+    if not 0 < r.real <= r.E:
+        raise BackendError(f"routing: {r.real} of {r.E} experts have matrices")
     _check(logits, "logits", torch.float32, (r.T, None))
     ld = logits.shape[1]
     if ld < r.E:
@@ -62,7 +70,7 @@ def route(logits, bias, routing, scores=False, groups=1, keep=1):
     lib.call("moe", "hb_moe_route", logits.data_ptr(), _ptr(bias), r.chosen.data_ptr(), r.weight.data_ptr(),
              r.counts.data_ptr(), r.order.data_ptr(), r.row_of.data_ptr(), r.tile_expert.data_ptr(),
              r.tile_row0.data_ptr(), r.tile_rows.data_ptr(), r.T, r.E, r.top, r.tiles, ld, 1 if scores else 0,
-             int(groups), int(keep), _stream())
+             int(groups), int(keep), r.real, 1 if score == "softmax" else 0, int(worth_top), 1 if renorm else 0, _stream())
 
 
 def gemm_plain(a, w, c, routing, gather):
@@ -70,7 +78,7 @@ def gemm_plain(a, w, c, routing, gather):
     gather (src = the pair's token) or [pairs, K]; c f32 [pairs, N]."""
     r = routing
     E, N, K = w.shape
-    _check(w, "w", None, (r.E, N, K))
+    _check(w, "w", None, (r.real, N, K))
     _check(a, "a", None, (r.T if gather else r.T * r.top, K))
     _check(c, "c", torch.float32, (r.T * r.top, N))
     lib.call("moe", "hb_moe_gemm_plain", a.data_ptr(), dtype_code(a), w.data_ptr(), dtype_code(w), c.data_ptr(),
@@ -90,9 +98,11 @@ def activate(gu, act, limit, alpha, shift=1.0):
              float(alpha), float(shift), _stream())
 
 
-def combine(y, routing, x, shared=None, gate=None):
+def combine(y, routing, x, shared=None, gate=None, identity=None):
     """x[t] += sum_j weight[t, j] * y[row of pair (t, j)]; y f32 [pairs, H], x f32 [T, H].
-    shared f32 [T, H] with gate = (f32 [T, ld], column): x[t] += sigmoid(gate[t, column]) * shared[t] as well."""
+    shared f32 [T, H] with gate = (f32 [T, ld], column): x[t] += sigmoid(gate[t, column]) * shared[t] as well.
+    identity [T, H] (float32 or bfloat16): the experts' input rows, which are the output of a pair whose expert has
+    no matrices (routing.real and beyond); needed where there are such experts."""
     r = routing
     H = x.shape[1]
     shared_ptr = gate_ptr = None
@@ -107,8 +117,13 @@ def combine(y, routing, x, shared=None, gate=None):
         shared_ptr, gate_ptr = shared.data_ptr(), rows.data_ptr() + 4 * column
     _check(y, "y", torch.float32, (r.T * r.top, H))
     _check(x, "x", torch.float32, (r.T, H))
+    if r.real < r.E and identity is None:
+        raise BackendError("moe combine: experts without matrices need the experts' input rows")
+    if identity is not None:
+        _check(identity, "identity", None, (r.T, H))
     lib.call("moe", "hb_moe_combine", y.data_ptr(), r.weight.data_ptr(), r.row_of.data_ptr(), x.data_ptr(), r.T,
-             r.top, H, shared_ptr, gate_ptr, gate_ld, _stream())
+             r.top, H, shared_ptr, gate_ptr, gate_ld, _ptr(identity) if r.real < r.E else None,
+             0 if identity is None else dtype_code(identity), r.chosen.data_ptr(), r.real, _stream())
 
 
 EPI_F32, EPI_BF16, EPI_GLU = 0, 1, 2
@@ -147,7 +162,7 @@ def grouped_mfma(a, lda, a_group_off, w, c, ldc, c_group_off, epi, routing=None,
     if routing is not None:
         r = routing
         rows_a, rows_c = (r.T if gather else r.T * r.top), r.T * r.top
-        if G != r.E:
+        if G != r.real:
             raise BackendError("grouped product: one matrix an expert")
         lists = (r.order.data_ptr(), r.top if gather else 0, r.tile_expert.data_ptr(), r.tile_row0.data_ptr(),
                  r.tile_rows.data_ptr(), r.tiles, 0, 0)

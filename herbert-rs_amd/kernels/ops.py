@@ -187,9 +187,11 @@ def qk_norm_rope_write(qkv, q_norm_w, k_norm_w, cos, sin, rot_dims, meta, cache,
              n_slices, stride, coef, every, _stream())
 
 
-def attention_plain(q, meta, cache, out, nq, nkv, hd, scale, window, sinks=None):
+def attention_plain(q, meta, cache, out, nq, nkv, hd, scale, window, sinks=None, chunk=None, softcap=None):
     """Causal (and windowed) attention of every token over its slot's pages. sinks f32 [nq]: the softmax's
-    denominator of head h also holds exp(sinks[h])."""
+    denominator of head h also holds exp(sinks[h]). chunk: a query sees the keys of its own chunk of that many
+    positions only (counted from the sequence's start; not together with a window). softcap: a scaled score s
+    becomes softcap tanh(s / softcap)."""
     T = q.shape[0]
     if sinks is not None:
         _check(sinks, "sinks", torch.float32, (nq,))
@@ -202,7 +204,7 @@ def attention_plain(q, meta, cache, out, nq, nkv, hd, scale, window, sinks=None)
              cache.v.data_ptr(), out.data_ptr(), dtype_code(q), meta.positions.data_ptr(),
              meta.seq_of.data_ptr(), meta.slots.data_ptr(), cache.page_table.data_ptr(),
              cache.page_table.shape[1], cache.page_size, T, nq, nkv, hd, float(scale),
-             int(window or 0), _ptr(sinks), _stream())
+             int(window or 0), _ptr(sinks), int(chunk or 0), float(softcap or 0.0), _stream())
 
 
 GLU_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
@@ -521,14 +523,16 @@ def normed_pair(a, wa, ca, b, wb, cb, out, eps, accumulate=False):
 
 
 def filter_norm_rotate_write(proj, taps, filter_state, q_norm_w, k_norm_w, rates, rot_dims, meta, cache, q_out,
-                             nq, nkv, dim, vdim, hd, eps):
+                             nq, nkv, dim, vdim, hd, eps, bias=None, head_norm=False):
     """The first columns of proj's rows (f32 [T, ld]) are [nq x dim queries | nkv x dim keys | nkv x vdim values]:
     filtered along time (taps f32 [C, K] with the slot's last inputs in filter_state f32 [slots, K - 1, C]; None:
     no filter), queries and keys each normed over the whole projection (weights [nq x dim], [nkv x dim]; None:
     no norm), neighbouring pairs of the first rot_dims entries of every head turned by position x rates (f64
     [rot_dims / 2]; None: no rotation); q to q_out [T, nq x hd], keys and values to the token's page, heads kept
     at hd with zeros beyond their own size. The filter's state is moved on too: by the kernel itself where every
-    sequence brings one token (meta.max_new), by the filter-state kernel afterwards otherwise."""
+    sequence brings one token (meta.max_new), by the filter-state kernel afterwards otherwise.
+    bias f32 [C]: added to the channels after the filter. head_norm: every query head and every key head is
+    normed by itself, with weights [dim] that all heads share."""
     T, ld = proj.shape
     C = (nq + nkv) * dim + nkv * vdim
     _check(proj, "proj", torch.float32, (T, ld))
@@ -538,10 +542,14 @@ def filter_norm_rotate_write(proj, taps, filter_state, q_norm_w, k_norm_w, rates
         _check(taps, "taps", torch.float32, (C, K))
         if K > 1:
             _check(filter_state, "filter_state", torch.float32, (None, K - 1, C))
+    if head_norm and (q_norm_w is None or k_norm_w is None):
+        raise BackendError("filtered attention: a norm a head needs its weights")
     if q_norm_w is not None:
-        _check(q_norm_w, "q_norm", torch.float32, (nq * dim,))
+        _check(q_norm_w, "q_norm", torch.float32, (dim if head_norm else nq * dim,))
     if k_norm_w is not None:
-        _check(k_norm_w, "k_norm", torch.float32, (nkv * dim,))
+        _check(k_norm_w, "k_norm", torch.float32, (dim if head_norm else nkv * dim,))
+    if bias is not None:
+        _check(bias, "bias", torch.float32, (C,))
     if rates is not None:
         _check(rates, "rates", torch.float64, (rot_dims // 2,))
     _check_paged(meta, cache, T)
@@ -556,11 +564,37 @@ def filter_norm_rotate_write(proj, taps, filter_state, q_norm_w, k_norm_w, rates
              meta.positions.data_ptr(), meta.seq_of.data_ptr(), meta.seq_starts.data_ptr(), meta.slots.data_ptr(),
              cache.page_table.data_ptr(), cache.page_table.shape[1], cache.page_size, q_out.data_ptr(),
              cache.k.data_ptr(), cache.v.data_ptr(), dtype_code(q_out), T, nq, nkv, dim, vdim, hd, float(eps),
-             int(meta.max_new), _stream())
+             int(meta.max_new), _ptr(bias), 1 if head_norm else 0, _stream())
     if K > 1 and meta.max_new != 1:
         _check(meta.slots, "slots", torch.int32, (meta.num_seqs,))
         lib.call("recurrent", "hb_filter_state", proj.data_ptr(), ld, filter_state.data_ptr(), meta.seq_starts.data_ptr(),
                  meta.slots.data_ptr(), meta.num_seqs, C, K, None, _stream())
+
+
+def add_bias(x, bias):
+    """x[t, :] += bias: x f32 [T, H], bias f32 [H]."""
+    T, H = x.shape
+    _check(x, "x", torch.float32, (T, H))
+    _check(bias, "bias", torch.float32, (H,))
+    lib.call("elementwise", "hb_add_bias", x.data_ptr(), bias.data_ptr(), T, H, _stream())
+
+
+def token_side(x, token_ids, table, col0, w_gate, w_proj, norm_w, eps):
+    """x += rmsnorm(W_proj (gelu_tanh(W_gate x) * table[token, col0 : col0 + D])) * norm_w, row by row and in
+    place: x f32 [T, H], token_ids int32 [T], table [V, ld], W_gate [D, H], W_proj [H, D] (one dtype), norm_w f32 [H]."""
+    T, H = x.shape
+    D = w_gate.shape[0]
+    _check(x, "x", torch.float32, (T, H))
+    _check(token_ids, "token_ids", torch.int32, (T,))
+    _check(table, "table", w_gate.dtype, (None, None))
+    _check(w_gate, "gate", None, (D, H))
+    _check(w_proj, "proj", w_gate.dtype, (H, D))
+    _check(norm_w, "norm", torch.float32, (H,))
+    if col0 < 0 or col0 + D > table.shape[1]:
+        raise BackendError("token input: the layer's columns lie outside the table's rows")
+    lib.call("elementwise", "hb_token_side", x.data_ptr(), token_ids.data_ptr(), table.data_ptr(), table.shape[1],
+             int(col0), w_gate.data_ptr(), w_proj.data_ptr(), dtype_code(w_gate), norm_w.data_ptr(), T, H, D, float(eps),
+             _stream())
 
 
 def gate_heads(attn, gate_rows, g_off, out, nq, hd, vdim):

@@ -11,13 +11,17 @@ MAX_TAPS = 16
 MAX_KEY_DIM = 256
 
 
-def conv_silu(proj, taps, conv_state, meta, out, n_unit, unit_dim, n_scaled, scale, unit_eps, n_plain, plain_dim):
-    """out[t, c] = silu(sum_j taps[c, j] * input[t - (K - 1) + j, c]) over the first C columns of proj
-    (f32 [T, ld]); inputs from before the step come from conv_state (f32 [slots, K - 1, C]), which is
+def conv_silu(proj, taps, conv_state, meta, out, n_unit, unit_dim, n_scaled, scale, unit_eps, n_plain, plain_dim,
+              col0=0, bias=None):
+    """out[t, c] = silu(sum_j taps[c, j] * input[t - (K - 1) + j, c]) over the C columns of proj (f32 [T, ld])
+    from col0 on; inputs from before the step come from conv_state (f32 [slots, K - 1, C]), which is
     then moved on. The first n_unit sections of unit_dim channels become unit vectors (the first
-    n_scaled of them times `scale`), the n_plain sections of plain_dim that follow stay as they are."""
+    n_scaled of them times `scale`), the n_plain sections of plain_dim that follow stay as they are (the last
+    of them may be shorter). bias f32 [C]: the sums start there."""
     T, ld = proj.shape
     C, K = taps.shape
+    if bias is not None:
+        _check(bias, "conv bias", torch.float32, (C,))
     _check(proj, "proj", torch.float32, (T, ld))
     _check(taps, "taps", torch.float32, (C, K))
     _check(conv_state, "conv_state", torch.float32, (None, max(K - 1, 1), C))
@@ -25,13 +29,51 @@ def conv_silu(proj, taps, conv_state, meta, out, n_unit, unit_dim, n_scaled, sca
     _check(meta.seq_of, "seq_of", torch.int32, (T,))
     _check(meta.seq_starts, "seq_starts", torch.int32, (meta.num_seqs + 1,))
     _check(meta.slots, "slots", torch.int32, (meta.num_seqs,))
-    if n_unit * unit_dim + n_plain * plain_dim != C or ld < C or not 1 <= K <= MAX_TAPS:
+    if n_unit * unit_dim + n_plain * plain_dim < C or col0 < 0 or ld < col0 + C or not 1 <= K <= MAX_TAPS:
         raise BackendError(f"conv: sections {n_unit} x {unit_dim} + {n_plain} x {plain_dim} do not fit {C} channels "
                            f"of {K} taps")
-    lib.call("recurrent", "hb_conv_silu", proj.data_ptr(), ld, taps.data_ptr(), conv_state.data_ptr(),
+    lib.call("recurrent", "hb_conv_silu", proj.data_ptr() + 4 * col0, ld, taps.data_ptr(), conv_state.data_ptr(),
              meta.seq_of.data_ptr(), meta.seq_starts.data_ptr(), meta.slots.data_ptr(), out.data_ptr(), T,
              meta.num_seqs, C, K, n_unit, unit_dim, n_scaled, float(scale), float(unit_eps), n_plain, plain_dim,
-             _stream())
+             None if bias is None else bias.data_ptr(), _stream())
+
+
+MAX_SSM_STATE = 256
+
+
+def ssm_scan(u, proj, dt_off, dt_bias, a_log, d_skip, state, meta, out, heads, groups, N, P):
+    """The state-space walk of every sequence of the step: u f32 [T, heads P + 2 groups N] (x, B, C as the
+    convolution left them), the step sizes' pre-activations in columns [dt_off, + heads) of proj (f32 [T, ld]);
+    dt = softplus(. + dt_bias), S <- exp(-exp(a_log) dt) S + dt B x^T, out = S^T C + d_skip x; state f32
+    [slots, heads, N, P] advanced in place, out f32 [T, heads P]."""
+    T = u.shape[0]
+    _check(u, "u", torch.float32, (T, heads * P + 2 * groups * N))
+    _check(proj, "proj", torch.float32, (T, None))
+    for t, name in ((dt_bias, "dt_bias"), (a_log, "A_log"), (d_skip, "D")):
+        _check(t, name, torch.float32, (heads,))
+    _check(state, "state", torch.float32, (None, heads, N, P))
+    _check(out, "out", torch.float32, (T, heads * P))
+    _check(meta.seq_starts, "seq_starts", torch.int32, (meta.num_seqs + 1,))
+    _check(meta.slots, "slots", torch.int32, (meta.num_seqs,))
+    if heads % groups or not 0 < N <= MAX_SSM_STATE or dt_off < 0 or dt_off + heads > proj.shape[1]:
+        raise BackendError(f"state-space walk: {heads} heads in {groups} groups, a state of {N} rows")
+    lib.call("recurrent", "hb_ssm_scan", u.data_ptr(), u.shape[1], proj.data_ptr(), proj.shape[1], int(dt_off),
+             dt_bias.data_ptr(), a_log.data_ptr(), d_skip.data_ptr(), state.data_ptr(), meta.seq_starts.data_ptr(),
+             meta.slots.data_ptr(), out.data_ptr(), meta.num_seqs, heads, groups, N, P, _stream())
+
+
+def gated_group_norm(o, proj, z_off, weight, out, parts, eps):
+    """out = v / rms(v) * weight with v = o * silu(proj[:, z_off ...]), the root mean square taken over each of
+    `parts` equal groups of a row by itself; o f32 [T, width], weight f32 [width], out in any dtype."""
+    T, width = o.shape
+    _check(o, "o", torch.float32, (T, width))
+    _check(proj, "proj", torch.float32, (T, None))
+    _check(weight, "weight", torch.float32, (width,))
+    _check(out, "out", None, (T, width))
+    if parts <= 0 or width % parts or z_off < 0 or z_off + width > proj.shape[1]:
+        raise BackendError(f"gated norm in groups: {width} columns in {parts} groups")
+    lib.call("recurrent", "hb_gated_group_norm", o.data_ptr(), proj.data_ptr(), proj.shape[1], int(z_off),
+             weight.data_ptr(), out.data_ptr(), dtype_code(out), T, width, int(parts), float(eps), _stream())
 
 
 def gated_delta(qkv, proj, b_off, a_off, a_log, dt_bias, state, meta, out, kv_heads, heads, D, V, decay=None,

@@ -1,4 +1,4 @@
 """Architectures: each module turns its typed configuration into a ModelSpec and registers itself."""
-from . import mefatar, modasun, qwen3, vipalorn
+from . import bozasun, mefatar, modasun, qwen3, vipalorn
 
-__all__ = ["mefatar", "modasun", "qwen3", "vipalorn"]
+__all__ = ["bozasun", "mefatar", "modasun", "qwen3", "vipalorn"]

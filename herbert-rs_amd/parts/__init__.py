@@ -2,7 +2,7 @@
 from .base import Part, Runtime, StepContext
 from .registry import CATEGORIES, build, register, registered
 from .spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
-from . import attention, block, delta, io, latent, linear_attention, lru, mlp, moe, norm, position, sides   # registers the built-in kinds
+from . import attention, block, delta, io, latent, linear_attention, lru, mlp, moe, norm, position, sides, ssm, token_input   # registers the built-in kinds
 
 __all__ = ["CATEGORIES", "LayerSpec", "ModelSpec", "Part", "PartSpec", "Runtime", "ScheduleEntry",
            "StepContext", "build", "register", "registered"]

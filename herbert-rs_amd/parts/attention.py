@@ -21,8 +21,11 @@ conv - 1 projected rows of a sequence are state beside its keys and values), `qk
 are normed over the whole projection at once, before they are split into heads, with a weight of that size),
 a position of the kind "rope_pairs" (neighbouring pairs turn), `sink` (the softmax's denominator of a head also
 holds exp(s_h), a stored number a head without key or value), `gate` (the joined heads times sigmoid(W_g y)
-before the output projection). Such a part filters, norms, rotates and writes the cache in one kernel of its
-own; rotation and values of another size than the keys go together there.
+before the output projection), `bias` (q, k, v and the output projection have biases), `chunk` (a query sees
+the keys of its own chunk of that many positions only, the chunks counted from the sequence's start),
+`softcap` (a scaled score s becomes softcap tanh(s / softcap) before the softmax). Such a part filters, norms
+(over the whole projection, or head by head with weights that all heads share), rotates and writes the cache in
+one kernel of its own; rotation and values of another size than the keys go together there.
 
 The kernels keep one head size for queries, keys and values. Where a model's
 key and value sizes differ, or where the matrix cores (heads of 32, 64, 128)
@@ -49,6 +52,11 @@ def _taps_init(shape, gen, device, std, norm_std):
     return 1.0 / shape[1] + 0.3 * torch.randn(shape, generator=gen, device=device, dtype=torch.float32)
 
 
+def _bias_init(shape, gen, device, std, norm_std):
+    """Biases of a random model: large enough beside the projections' sums that leaving one out shows."""
+    return 0.5 * torch.randn(shape, generator=gen, device=device, dtype=torch.float32)
+
+
 def _sink_init(shape, gen, device, std, norm_std):
     """Sinks of a random model: around zero, so that they take a visible share of a short row's weight."""
     return torch.randn(shape, generator=gen, device=device, dtype=torch.float32)
@@ -60,9 +68,10 @@ class Attention(Part):
 
     def __init__(self, hidden_size, num_heads, num_kv_heads, head_dim, eps, position, names,
                  qk_norm=True, window=None, scale=None, shared=None, reads_cache_only=False,
-                 value_dim=None, q_temp=None, conv=None, sink=False, gate=False):
+                 value_dim=None, q_temp=None, conv=None, sink=False, gate=False, bias=False, chunk=None,
+                 softcap=None):
         """names: dict with q, k, v, o (and q_norm, k_norm when qk_norm is True or "whole"; q_conv, k_conv, v_conv
-        with conv; sink with sink; g with gate) -> tensor names.
+        with conv; sink with sink; g with gate; q_bias, k_bias, v_bias, o_bias with bias) -> tensor names.
         qk_norm: True (a weight [head_dim] each for queries and keys), "plain" (no weights), "whole" (over all
         heads of a token at once, weights of that size) or False.
         conv: taps of a filter along time on queries, keys and values (None: none).
@@ -90,17 +99,23 @@ class Attention(Part):
         self.position = shared.position(position)
         self.qkv = self.o = self.q_norm_w = self.k_norm_w = None
         self.taps = int(conv) if conv else 0
-        self.sink, self.gate = bool(sink), bool(gate)
-        self.sink_w = self.taps_w = None
+        self.sink, self.gate, self.bias = bool(sink), bool(gate), bool(bias)
+        self.chunk = int(chunk) if chunk else None
+        self.softcap = float(softcap) if softcap else None
+        if self.chunk is not None and (self.chunk <= 0 or self.window):
+            raise ValueError("chunk is a positive number of positions and does not go with a window")
+        if self.softcap is not None and self.softcap <= 0:
+            raise ValueError("softcap must be positive")
+        self.sink_w = self.taps_w = self.bias_w = self.o_bias_w = None
         # the form with a kernel of its own before the attention (see the module's text)
-        self.prepared = bool(self.taps or self.sink or self.gate or qk_norm == "whole"
-                             or hasattr(self.position, "pair_rates"))
+        self.prepared = bool(self.taps or self.sink or self.gate or qk_norm == "whole" or self.bias or self.chunk
+                             or self.softcap or hasattr(self.position, "pair_rates"))
         if self.prepared:
-            if self.reads_cache_only or self.q_temp is not None or qk_norm in (True, "plain") or \
+            if self.reads_cache_only or self.q_temp is not None or qk_norm == "plain" or \
                     self.position.rotation() is not None:
-                raise ValueError("a filter, a norm over the whole projection, a rotation of pairs, a sink or a gate "
-                                 "go with a cache of the part's own, no per-head norm, no growing query and no "
-                                 "rotation of halves")
+                raise ValueError("a filter, a norm over the whole projection, a rotation of pairs, a sink, a gate, "
+                                 "biases, chunks or capped scores go with a cache of the part's own, no norm without "
+                                 "weights, no growing query and no rotation of halves")
             if self.taps > recurrent.MAX_TAPS:
                 raise ValueError(f"the filter takes up to {recurrent.MAX_TAPS} taps, not {self.taps}")
             self.stores_fresh_rows = True        # its output projection stores into rows that hold nothing yet
@@ -141,6 +156,11 @@ class Attention(Part):
             needs[n["sink"]] = TensorNeed((self.nq,), "bias", _sink_init)
         if self.gate:
             needs[n["g"]] = TensorNeed((self.nq * self.vdim, W))
+        if self.bias:
+            needs[n["q_bias"]] = TensorNeed((self.nq * self.dim,), "bias", _bias_init)
+            needs[n["k_bias"]] = TensorNeed((self.nkv * self.dim,), "bias", _bias_init)
+            needs[n["v_bias"]] = TensorNeed((self.nkv * self.vdim,), "bias", _bias_init)
+            needs[n["o_bias"]] = TensorNeed((W,), "bias", _bias_init)
         if not self.reads_cache_only:
             needs[n["k"]] = TensorNeed((self.nkv * self.dim, W))
             needs[n["v"]] = TensorNeed((self.nkv * self.vdim, W))
@@ -200,9 +220,13 @@ class Attention(Part):
         self.qkv = Linear(rt.weight(torch.cat(rows, 0)), scratch=rt.scratch)
         self.proj_width = self.channels + (self.nq * self.vdim if self.gate else 0)
         self.o = Linear(rt.weight(tensors[n["o"]]), scratch=rt.scratch)
-        if self.qk_norm == "whole":
+        if self.qk_norm in ("whole", True):
             self.q_norm_w = rt.weight(tensors[n["q_norm"]], matrix=False)
             self.k_norm_w = rt.weight(tensors[n["k_norm"]], matrix=False)
+        if self.bias:
+            self.bias_w = torch.cat([rt.weight(tensors[n[k]], matrix=False) for k in ("q_bias", "k_bias", "v_bias")],
+                                    0).contiguous()
+            self.o_bias_w = rt.weight(tensors[n["o_bias"]], matrix=False)
         if self.taps:
             self.taps_w = torch.cat([rt.weight(tensors[n[k]], matrix=False) for k in ("q_conv", "k_conv", "v_conv")],
                                     0).contiguous()
@@ -219,13 +243,18 @@ class Attention(Part):
         state = ctx.cache.state_views(ctx.cache_entry)[0] if self.taps > 1 else None
         rates, rot_dims = self.position.pair_rates() if hasattr(self.position, "pair_rates") else (None, 0)
         ops.filter_norm_rotate_write(proj, self.taps_w, state, self.q_norm_w, self.k_norm_w, rates, rot_dims, ctx.meta,
-                                     kv, q, self.nq, self.nkv, self.dim, self.vdim, self.hd, self.eps)
+                                     kv, q, self.nq, self.nkv, self.dim, self.vdim, self.hd, self.eps, bias=self.bias_w,
+                                     head_norm=self.qk_norm is True)
         attn = rt.buffer("attn", (T, self.q_dim))
         self.attend(ctx, q, kv, attn)
         # the heads leave at their own size, each entry times its gate
-        gated = rt.buffer("attn_gated", (T, self.nq * self.vdim))
-        ops.gate_heads(attn, proj if self.gate else None, self.channels, gated, self.nq, self.hd, self.vdim)
+        gated = attn
+        if self.gate or self.hd != self.vdim:
+            gated = rt.buffer("attn_gated", (T, self.nq * self.vdim))
+            ops.gate_heads(attn, proj if self.gate else None, self.channels, gated, self.nq, self.hd, self.vdim)
         self.o.forward(gated, x, accumulate=ctx.adds_to(x))
+        if self.o_bias_w is not None:
+            ops.add_bias(x, self.o_bias_w)
 
     def load(self, tensors, rt):
         if self.prepared:
@@ -323,6 +352,7 @@ class Attention(Part):
         if q.dtype == torch.bfloat16:
             if mfma.attention_supported(q, kv, self.nq, self.nkv, self.hd):
                 mfma.attention(q, ctx.meta, kv, out, self.nq, self.nkv, self.hd, scale, self.window,
-                               scratch=ctx.rt.scratch, sinks=self.sink_w)
+                               scratch=ctx.rt.scratch, sinks=self.sink_w, chunk=self.chunk, softcap=self.softcap)
                 return
-        ops.attention_plain(q, ctx.meta, kv, out, self.nq, self.nkv, self.hd, scale, self.window, sinks=self.sink_w)
+        ops.attention_plain(q, ctx.meta, kv, out, self.nq, self.nkv, self.hd, scale, self.window, sinks=self.sink_w,
+                            chunk=self.chunk, softcap=self.softcap)

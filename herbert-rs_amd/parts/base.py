@@ -62,6 +62,7 @@ class Runtime:
         self._views = {}         # (name, dtype, shape) -> the view of the buffer that was handed out last
         self._outgrown = []      # never freed: a captured graph may hold their addresses
         self._scratch = None
+        self._shared = {}        # (tensor name, matrix) -> a stored tensor that several parts read, converted once
 
     @property
     def scratch(self):
@@ -106,6 +107,14 @@ class Runtime:
             self._views.clear()
         view = self._views[(name, dtype, shape)] = buf[:n].view(*shape)
         return view
+
+    def shared_weight(self, name, t, matrix=True):
+        """`weight(t)` for a stored tensor that several parts read (a table with a part for every layer): converted
+        and kept once under its name."""
+        kept = self._shared.get((name, matrix))
+        if kept is None:
+            kept = self._shared[(name, matrix)] = self.weight(t, matrix)
+        return kept
 
     def weight(self, t, matrix=True):
         """A stored tensor as the kernels read it: matrices in the compute dtype, scales in float32."""

@@ -10,14 +10,16 @@ take x as it is, and each norm comes after its sum.
 arrangement of the reference's two-norm layer
 (crates/backends/backend_common/src/generic_layer.rs:1149-1151, 1234-1236,
 1246-1248, 1272-1274). With `branch_scale` (not in the reference) each branch is multiplied, channel by
-channel, by a learned factor before it joins x, and the layer may have no feed-forward.
+channel, by a learned factor before it joins x, and the layer may have no feed-forward. With `token_input` (not in
+the reference either) a part of the category "token_input" adds to x after the layer's other parts, from x itself
+and the tokens' ids; such a layer may have no feed-forward either.
 """
 import torch
 
 from ..kernels import ops
 from ..weights import TensorNeed
 from .base import Part
-from .registry import register
+from .registry import build, register
 
 
 class ChannelScale(Part):
@@ -42,12 +44,17 @@ class PreNormBlock(Part):
 
     norm_roles = ("input", "post_mixer")
 
-    def __init__(self, mixer, feed_forward, norms, branch_scale=None):
+    def __init__(self, mixer, feed_forward, norms, branch_scale=None, token_input=None):
         """branch_scale: None, or {"size": the model's width, "mixer": tensor name, "feed_forward": tensor name}:
         each branch times a stored factor a channel before the sum. Such a block's parts add to float32 rows
         of their own; the kernel of the norm that follows adds them, scaled, to x on its way (the last
         branch of a layer is left for the next layer's first norm, if that is such a block too). Only such
-        a block may do without a feed-forward."""
+        a block, or one with a token input, may do without a feed-forward.
+        token_input: None, or the PartSpec of a part of the category "token_input", whose forward(ctx, x) adds to x
+        after the mixer and the feed-forward."""
+        self.token_input = None if token_input is None else build("token_input", token_input)
+        if self.token_input is not None and branch_scale is not None:
+            raise ValueError("prenorm block: a token input does not go with scaled branches")
         self.mixer = mixer
         self.feed_forward = feed_forward
         self.norms = norms
@@ -56,8 +63,9 @@ class PreNormBlock(Part):
             self.scales = {"mixer": ChannelScale(branch_scale["size"], branch_scale["mixer"])}
             if feed_forward is not None:
                 self.scales["feed_forward"] = ChannelScale(branch_scale["size"], branch_scale["feed_forward"])
-        elif feed_forward is None:
-            raise ValueError("prenorm block: only a block with scaled branches may do without a feed-forward")
+        elif feed_forward is None and self.token_input is None:
+            raise ValueError("prenorm block: only a block with scaled branches or a token input may do without a "
+                             "feed-forward")
         missing = [r for r in self.norm_roles[:1 if feed_forward is None else 2] if r not in norms]
         if missing:
             raise ValueError(f"prenorm block needs norms {missing}")
@@ -72,6 +80,8 @@ class PreNormBlock(Part):
             parts += [self.norms["post_mixer"], self.feed_forward]
         if self.scales is not None:
             parts += list(self.scales.values())
+        if self.token_input is not None:
+            parts.append(self.token_input)
         return parts
 
     def first_norm(self):
@@ -115,9 +125,16 @@ class PreNormBlock(Part):
         if self.scales is not None:
             self._forward_scaled(ctx, x)
             return
-        after = ctx.norm_after_block
-        self._run(ctx, x, self.norms["input"], self.mixer, (self.norms["post_mixer"], ctx.entry))
-        self._run(ctx, x, self.norms["post_mixer"], self.feed_forward, after)
+        # (x changes once more after the parts where the block has a token input: nobody prepares the next norm then)
+        after = ctx.norm_after_block if self.token_input is None else None
+        if self.feed_forward is None:
+            self._run(ctx, x, self.norms["input"], self.mixer, after)
+        else:
+            self._run(ctx, x, self.norms["input"], self.mixer, (self.norms["post_mixer"], ctx.entry))
+            self._run(ctx, x, self.norms["post_mixer"], self.feed_forward, after)
+        if self.token_input is not None:
+            ctx.handed = ctx.norm_ahead = ctx.left = None
+            self.token_input.forward(ctx, x)
 
     @staticmethod
     def _run(ctx, x, norm, part, ahead):

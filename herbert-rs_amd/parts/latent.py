@@ -11,6 +11,12 @@ no values beside them. The kernels never build a head's keys or values: the quer
 W_uk,n^T first (kv_rank numbers), scores and weighted sums then run on the cached rows themselves,
 one shared "key head" for all query heads, and the summed latents go through W_uv,n afterwards.
 Scores, softmax and the weighted sums are float32 in either mode.
+
+Two parameters change the form. `gate="elementwise"`: W_g has a row for every entry of the joined heads, and
+each entry is multiplied by the sigmoid of its own (after W_uv, in a kernel of its own). `pairs=True`: the
+rotation turns neighbouring entries (2i, 2i + 1) instead of entries half the rotated size apart; since a score
+only ever sees the rotated parts of a query and a key together, the rows of W_q's and W_dkv's rotated parts
+are put into the order (even entries, then odd ones) when they are loaded, and the kernels rotate as they do.
 """
 import torch
 
@@ -27,7 +33,8 @@ class LatentAttention(Part):
     graph_safe = True
     stores_fresh_rows = True     # its output projection stores into rows that hold nothing yet (StepContext.adds_to)
 
-    def __init__(self, hidden_size, heads, dim, rot_dim, vdim, kv_rank, scale, eps, position, names, shared=None):
+    def __init__(self, hidden_size, heads, dim, rot_dim, vdim, kv_rank, scale, eps, position, names, shared=None,
+                 gate="head", pairs=False):
         """names: q, dkv, dkv_norm, uk, uv, g (None: no output gate), o -> tensor names. position: the
         spec of a rotation (its rotary_dims <= rot_dim entries of the rotated part are rotated)."""
         self.hidden_size, self.heads = int(hidden_size), int(heads)
@@ -35,6 +42,9 @@ class LatentAttention(Part):
         self.scale, self.eps = float(scale), float(eps)
         self.names = dict(names)
         self.position = shared.position(position)
+        if gate not in ("head", "elementwise"):
+            raise ValueError(f"gate is 'head' or 'elementwise', not {gate!r}")
+        self.gate_kind, self.pairs = gate, bool(pairs)
         if self.rank > latent.MAX_RANK or self.rot_dim > latent.MAX_ROT:
             raise ValueError(f"the latent attention's kernels take a latent of up to {latent.MAX_RANK} + "
                              f"{latent.MAX_ROT}, not {self.rank} + {self.rot_dim}")
@@ -49,7 +59,7 @@ class LatentAttention(Part):
                  n["dkv_norm"]: TensorNeed((self.rank,), "scale"), n["uk"]: TensorNeed((H * self.dim, self.rank)),
                  n["uv"]: TensorNeed((H * self.vdim, self.rank)), n["o"]: TensorNeed((W, H * self.vdim))}
         if n.get("g"):
-            needs[n["g"]] = TensorNeed((H, W))
+            needs[n["g"]] = TensorNeed((H * self.vdim if self.gate_kind == "elementwise" else H, W))
         return needs
 
     def cache_need(self):
@@ -57,14 +67,30 @@ class LatentAttention(Part):
 
     def load(self, tensors, rt):
         n, H = self.names, self.heads
-        rows = [tensors[n["q"]].to(rt.device), tensors[n["dkv"]].to(rt.device)]
+        rot = self.position.rotation_rates()
+        self.inv_freq, self.rot_dims = (None, 0) if rot is None else rot
+        if self.rot_dims > self.rot_dim:
+            raise ValueError(f"{self.rot_dims} rotated entries do not fit the rotated part of {self.rot_dim}")
+        wq, wdkv = tensors[n["q"]].to(rt.device), tensors[n["dkv"]].to(rt.device)
+        if self.pairs and self.rot_dims:
+            # the rotated entries in the order (even, odd): the kernels' rotation of entries half the size apart
+            # then turns what were neighbours
+            order = torch.cat([torch.arange(0, self.rot_dims, 2), torch.arange(1, self.rot_dims, 2),
+                               torch.arange(self.rot_dims, self.rot_dim)]).to(rt.device)
+            per = self.dim + self.rot_dim
+            q_rows = torch.cat([torch.cat([torch.arange(self.dim, device=rt.device), self.dim + order]) + h * per
+                                for h in range(H)])
+            wq = wq[q_rows]
+            wdkv = wdkv[torch.cat([torch.arange(self.rank, device=rt.device), self.rank + order])]
+        rows = [wq, wdkv]
         self.gated = bool(n.get("g"))
         if self.gated:
             rows.append(tensors[n["g"]].to(rt.device))
         # one projection [q | latent and shared key part | gate]
         self.proj = Linear(rt.weight(torch.cat(rows, 0)), scratch=rt.scratch)
         self.q_width = H * (self.dim + self.rot_dim)
-        self.width = self.q_width + self.row + (H if self.gated else 0)
+        self.gate_width = 0 if not self.gated else H * self.vdim if self.gate_kind == "elementwise" else H
+        self.width = self.q_width + self.row + self.gate_width
         self.norm_w = rt.weight(tensors[n["dkv_norm"]], matrix=False)
         # W_uk a head, transposed: [H, rank, dim], so that q' = W_uk,n^T q_n is a product with rows of k = dim
         uk = rt.weight(tensors[n["uk"]]).view(H, self.dim, self.rank)
@@ -76,10 +102,6 @@ class LatentAttention(Part):
                       and moe.mfma_takes(self.rank, H * self.rank, self.rank, self.vdim))
         if self.cores:
             self.uk_t, self.uv = moe.pack_grouped(self.uk_t), moe.pack_grouped(self.uv)
-        rot = self.position.rotation_rates()
-        self.inv_freq, self.rot_dims = (None, 0) if rot is None else rot
-        if self.rot_dims > self.rot_dim:
-            raise ValueError(f"{self.rot_dims} rotated entries do not fit the rotated part of {self.rot_dim}")
 
     def forward(self, ctx, y, x):
         rt, H = ctx.rt, self.heads
@@ -100,7 +122,7 @@ class LatentAttention(Part):
             ops.gemm_plain_batched(proj, self.uk_t, q_full, T, self.rank, self.dim, self.width, self.dim,
                                    H * self.row, H, self.dim + self.rot_dim, self.rank * self.dim, self.row)
         mixed = rt.buffer("latent_mixed", (T, H * self.rank))
-        gate = proj if self.gated else None
+        gate = proj if self.gated and self.gate_kind == "head" else None
         if latent.mfma_takes(kv, self.rank, self.rot_dim):
             latent.latent_attention_mfma(q_full, ctx.meta, kv, mixed, gate, self.q_width + self.row, H, self.rank,
                                          self.rot_dim, self.scale, rt.buffer)
@@ -114,6 +136,10 @@ class LatentAttention(Part):
         else:
             ops.gemm_plain_batched(mixed, self.uv, attn, T, self.vdim, self.rank, H * self.rank, self.rank,
                                    H * self.vdim, H, self.rank, self.vdim * self.rank, self.vdim)
+        if self.gated and self.gate_kind == "elementwise":
+            gated = rt.buffer("latent_gated", (T, H * self.vdim))
+            ops.gate_heads(attn, proj, self.q_width + self.row, gated, H, self.vdim, self.vdim)
+            attn = gated
         adds = ctx.adds_to(x)
         left = ctx.leave_norm(self.o, x) if adds else None
         self.o.forward(attn, x, accumulate=adds, leave=None if left is None else left.leave())

@@ -12,7 +12,11 @@ vector) and only within the `keep` best of `groups` equal groups of neighbouring
 the two highest of its selection values, added; the weights are the chosen experts' s over their sum (+ 1e-20).
 `activation="silu"`: an expert is W_down (silu(W_gate y) (W_up y)), nothing clamped. `shared_expert`: one more
 expert of that form and a width of its own that every token takes, its output times sigmoid(w_sg . y) (one
-number a token) added to the routed experts' sum.
+number a token) added to the routed experts' sum. With routing "scores" three more: `scoring="softmax"` (s is the
+softmax of z over all experts instead of its sigmoids), `group_worth=1` (a group is worth its highest selection
+value alone), `renormalize=False` (the weights are the chosen experts' s as they are). `identity`: so many
+further outputs of the router, behind the experts', stand for experts without matrices, whose output is their
+input; they are scored, grouped and chosen with the others.
 """
 import math
 
@@ -36,7 +40,8 @@ class RoutedExperts(Part):
     graph_safe = True
 
     def __init__(self, hidden_size, intermediate_size, experts, top, names, limit=None, alpha=GATE_ALPHA, shared=None,
-                 routing="softmax", groups=1, keep=1, activation="clamped", shared_expert=None):
+                 routing="softmax", groups=1, keep=1, activation="clamped", shared_expert=None, scoring="sigmoid",
+                 group_worth=2, renormalize=True, identity=0):
         """names: router, router_bias (None: none; with routing "scores" it is the correction of the choice),
         and gate, up, down as patterns with {e} for the expert's number.
         shared_expert: None or {"intermediate_size": .., "names": {gate, up, down, sg}}."""
@@ -46,6 +51,13 @@ class RoutedExperts(Part):
             raise ValueError(f"routing is 'softmax' or 'scores' and activation 'clamped' or 'silu', not {routing!r} "
                              f"and {activation!r}")
         self.routing, self.groups, self.keep = routing, int(groups), int(keep)
+        if scoring not in ("sigmoid", "softmax") or group_worth not in (1, 2):
+            raise ValueError(f"scoring is 'sigmoid' or 'softmax' and a group is worth its top 1 or 2, not {scoring!r}, {group_worth!r}")
+        self.scoring, self.group_worth, self.renormalize, self.identity = scoring, int(group_worth), bool(renormalize), int(identity)
+        if routing != "scores" and (scoring != "sigmoid" or group_worth != 2 or not renormalize or self.identity):
+            raise ValueError("softmax scores, a group's worth, weights as they are and experts without matrices go with routing 'scores'")
+        if self.identity < 0 or (self.identity and shared_expert is not None):
+            raise ValueError("experts without matrices: a count of zero or more, and no shared expert beside them")
         if activation == "silu":
             self.limit, self.alpha, self.shift = math.inf, 1.0, 0.0
         else:
@@ -53,21 +65,26 @@ class RoutedExperts(Part):
                 raise ValueError("the clamped activation needs its limit")
             self.limit, self.alpha, self.shift = float(limit), float(alpha), 1.0
         self.names = dict(names)
-        if not 0 < self.top <= self.experts or self.experts > moe.MAX_EXPERTS:
-            raise ValueError(f"{self.top} of {self.experts} experts (the router takes up to {moe.MAX_EXPERTS})")
-        if routing == "scores" and (self.groups <= 0 or self.experts % self.groups or not 0 < self.keep <= self.groups
-                                    or self.top > self.keep * (self.experts // self.groups)):
+        if not 0 < self.top <= self.routed or self.routed > moe.MAX_EXPERTS:
+            raise ValueError(f"{self.top} of {self.routed} experts (the router takes up to {moe.MAX_EXPERTS})")
+        if routing == "scores" and (self.groups <= 0 or self.routed % self.groups or not 0 < self.keep <= self.groups
+                                    or self.top > self.keep * (self.routed // self.groups)):
             raise ValueError(f"{self.top} experts cannot come from {self.keep} of {self.groups} groups of "
-                             f"{self.experts} experts")
+                             f"{self.routed} experts")
         self.shared_expert = None
         if shared_expert is not None:
             self.shared_expert = (int(shared_expert["intermediate_size"]), dict(shared_expert["names"]))
 
+    @property
+    def routed(self):
+        """Outputs of the router: the experts and, behind them, the experts without matrices."""
+        return self.experts + self.identity
+
     def tensor_needs(self):
         n, W, F = self.names, self.hidden_size, self.inter
-        needs = {n["router"]: TensorNeed((self.experts, W))}
+        needs = {n["router"]: TensorNeed((self.routed, W))}
         if n.get("router_bias"):
-            needs[n["router_bias"]] = TensorNeed((self.experts,), "bias", _bias_init)
+            needs[n["router_bias"]] = TensorNeed((self.routed,), "bias", _bias_init)
         for e in range(self.experts):
             needs[n["gate"].format(e=e)] = TensorNeed((F, W))
             needs[n["up"].format(e=e)] = TensorNeed((F, W))
@@ -116,13 +133,14 @@ class RoutedExperts(Part):
 
     def forward(self, ctx, y, x):
         rt = ctx.rt
-        T, E, top, F = y.shape[0], self.experts, self.top, self.inter
+        T, E, top, F = y.shape[0], self.routed, self.top, self.inter
         logits = rt.buffer("moe_logits", (T, self.router_width), torch.float32)
         self.router.forward(y, logits)          # float32 sums of the rows' products with the router's matrix
         routing = moe.Routing(rt.buffer("moe_ints", (moe.Routing.ints_needed(T, E, top),), torch.int32),
-                              rt.buffer("moe_weight", (T, top), torch.float32), T, E, top)
+                              rt.buffer("moe_weight", (T, top), torch.float32), T, E, top, real=self.experts)
         if self.routing == "scores":
-            moe.route(logits, self.router_bias, routing, scores=True, groups=self.groups, keep=self.keep)
+            moe.route(logits, self.router_bias, routing, scores=True, groups=self.groups, keep=self.keep,
+                      score=self.scoring, worth_top=self.group_worth, renorm=self.renormalize)
         else:
             moe.route(logits, self.router_bias, routing)
         shared = None
@@ -149,4 +167,5 @@ class RoutedExperts(Part):
             moe.gemm_plain(y, self.gate_up, gu, routing, gather=True)
             moe.activate(gu, act, self.limit, self.alpha, self.shift)
             moe.gemm_plain(act, self.down, out, routing, gather=False)
-        moe.combine(out, routing, x, shared=shared, gate=None if shared is None else (logits, E))
+        moe.combine(out, routing, x, shared=shared, gate=None if shared is None else (logits, E),
+                    identity=y if self.identity else None)

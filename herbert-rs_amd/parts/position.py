@@ -96,13 +96,19 @@ class RotaryPairs(Part):
     a position's angle, its sine and its cosine itself, so no table bounds the positions.
     scaling = (factor, low, high, original): a rate whose wavelength 2 pi / rate lies beyond original / low is
     divided by factor, one under original / high stays, and between the two, with
-    s = (original / wavelength - low) / (high - low), the rate is (1 - s) rate / factor + s rate."""
+    s = (original / wavelength - low) / (high - low), the rate is (1 - s) rate / factor + s rate.
+    scaling = ("linear", factor): every rate is divided by factor."""
     graph_safe = True
 
     def __init__(self, theta, rotary_dims, scaling=None):
         if rotary_dims % 2 or rotary_dims <= 0:
             raise ValueError("rotary_dims must be even and positive")
         self.theta, self.rotary_dims = float(theta), int(rotary_dims)
+        self.linear = None
+        if scaling is not None and scaling[0] == "linear":
+            self.linear, scaling = float(scaling[1]), None
+            if self.linear <= 0:
+                raise ValueError("the rates' divisor must be positive")
         self.scaling = None if scaling is None else tuple(float(v) for v in scaling)
         self.rates = None
 
@@ -110,6 +116,8 @@ class RotaryPairs(Part):
         rates = []
         for i in range(self.rotary_dims // 2):
             rate = self.theta ** (-2.0 * i / self.rotary_dims)
+            if self.linear is not None:
+                rate = rate / self.linear
             if self.scaling is not None:
                 factor, low, high, original = self.scaling
                 wavelength = 2.0 * math.pi / rate

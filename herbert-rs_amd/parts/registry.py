@@ -2,12 +2,13 @@
 
 A part class is registered with `@register(category, kind)` and built with
 `build(category, spec, **context)`. The categories are "mixer",
-"feed_forward", "norm", "position", "block", "embedding" and "head"; a test
+"feed_forward", "norm", "position", "block", "embedding", "head" and "token_input"
+(what a block may add to the residual stream from the tokens' ids after its parts); a test
 or a user may add kinds without touching this package.
 """
 from ..errors import ConfigError
 
-CATEGORIES = ("mixer", "feed_forward", "norm", "position", "block", "embedding", "head")
+CATEGORIES = ("mixer", "feed_forward", "norm", "position", "block", "embedding", "head", "token_input")
 _REGISTRY = {c: {} for c in CATEGORIES}
 
 
