@@ -12,7 +12,7 @@ arrangement of the reference's two-norm layer
 1246-1248, 1272-1274). With `branch_scale` (not in the reference) each branch is multiplied, channel by
 channel, by a learned factor before it joins x, and the layer may have no feed-forward. With `token_input` (not in
 the reference either) a part of the category "token_input" adds to x after the layer's other parts, from x itself
-and the tokens' ids; such a layer may have no feed-forward either.
+and the tokens' ids. A layer may have no feed-forward.
 """
 import torch
 
@@ -49,7 +49,7 @@ class PreNormBlock(Part):
         each branch times a stored factor a channel before the sum. Such a block's parts add to float32 rows
         of their own; the kernel of the norm that follows adds them, scaled, to x on its way (the last
         branch of a layer is left for the next layer's first norm, if that is such a block too). Only such
-        a block, or one with a token input, may do without a feed-forward.
+        A block may do without a feed-forward (the reference's layers all have one).
         token_input: None, or the PartSpec of a part of the category "token_input", whose forward(ctx, x) adds to x
         after the mixer and the feed-forward."""
         self.token_input = None if token_input is None else build("token_input", token_input)
@@ -63,9 +63,6 @@ class PreNormBlock(Part):
             self.scales = {"mixer": ChannelScale(branch_scale["size"], branch_scale["mixer"])}
             if feed_forward is not None:
                 self.scales["feed_forward"] = ChannelScale(branch_scale["size"], branch_scale["feed_forward"])
-        elif feed_forward is None and self.token_input is None:
-            raise ValueError("prenorm block: only a block with scaled branches or a token input may do without a "
-                             "feed-forward")
         missing = [r for r in self.norm_roles[:1 if feed_forward is None else 2] if r not in norms]
         if missing:
             raise ValueError(f"prenorm block needs norms {missing}")

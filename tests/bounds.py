@@ -33,9 +33,10 @@ F32_ABS = 1e-4
 #  configurations, the same and a float32 stream that is normed after every sum; "mef": the Mefatar
 #  configurations, whose stream, scores, recurrences and gates stay float32: worst seen 0.04 to 0.08 for most, 0.10
 #  to 0.11 on single rows of the narrowest (widths of 64 and 72 through seven to nine layer runs, vocabularies of
-#  96 to 320), which is why its model-level tests let one row in fifty pass the bound by half.)
-BF16_REL_L2 = {"mef": 0.03, "mod": 0.03, "vip": 0.03, "A": 0.012, "B": 0.018, "C": 0.018, "D": 0.02, "F": 0.02, "wide": 0.02, "odd": 0.02, "random": 0.02, "long": 0.025, "deep": 0.02}
-BF16_REL_RMS = {"mef": 0.1, "mod": 0.1, "vip": 0.1, "A": 0.04, "B": 0.05, "C": 0.05, "D": 0.05, "F": 0.05, "wide": 0.08, "odd": 0.04, "random": 0.06, "long": 0.08, "deep": 0.08}
+#  96 to 320), which is why its model-level tests let one row in fifty pass the bound by half; "boz": the Bozasun
+#  configurations, whose stream, scores, routing and state stay float32.)
+BF16_REL_L2 = {"boz": 0.03, "mef": 0.03, "mod": 0.03, "vip": 0.03, "A": 0.012, "B": 0.018, "C": 0.018, "D": 0.02, "F": 0.02, "wide": 0.02, "odd": 0.02, "random": 0.02, "long": 0.025, "deep": 0.02}
+BF16_REL_RMS = {"boz": 0.1, "mef": 0.1, "mod": 0.1, "vip": 0.1, "A": 0.04, "B": 0.05, "C": 0.05, "D": 0.05, "F": 0.05, "wide": 0.08, "odd": 0.04, "random": 0.06, "long": 0.08, "deep": 0.08}
 
 
 def rel_rms_error(got, ref):
@@ -53,7 +54,7 @@ def close(got, ref, dtype, config, label=None):
         observe(f"float32 {config} {label or ''} abs", err)
         return err <= F32_ABS, err
     ok = rel <= BF16_REL_RMS[config] and rel_l2 <= BF16_REL_L2[config]
-    if ok or config not in ("vip", "mod"):        # (of that family's rows a few may be off for a reason that is no rounding: the worst of the others is what counts)
+    if ok or config not in ("vip", "mod", "boz"):        # (of that family's rows a few may be off for a reason that is no rounding: the worst of the others is what counts)
         observe(f"bfloat16 {config} {label or ''} max / rms", rel)
         observe(f"bfloat16 {config} {label or ''} rms / rms", rel_l2)
     return ok, max(rel, rel_l2)
