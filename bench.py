@@ -21,7 +21,7 @@ step is what the generation loop does for a token: the step function (a HIP-grap
 greedy choice on the GPU, and the chosen tokens read by the host, which as in that loop reads
 the tokens of a step while the next step, fed from the GPU, already runs.
 
-`--workload vipalorn|modasun|mefatar --size small|medium|wide` measures one of the other designs instead (random weights at
+`--workload vipalorn|modasun|mefatar|bozasun --size small|medium|wide` measures one of the other designs instead (random weights at
 sizes that resemble a real model's layers) beside the closest other model at equal size, through the generation
 loop; the default workload and its JSON line stay as they are.
 """
@@ -206,9 +206,32 @@ def mefatar_configs(size):
     return mef, modasun_configs(size)[0]
 
 
+def bozasun_configs(size):
+    """(Bozasun config dict, Vipalorn config dict) of one size: of every four layers two state-space layers (twice
+    the model's width inside, heads of 64 columns, a state of 128 rows, eight groups, four taps), one attention
+    over chunks of 2,048 positions (biases, a norm a head, the whole head rotated at an eighth of the rates, scores
+    capped at 30) and one latent attention with a gate an entry; every layer with experts chosen by softmax scores
+    within two of four groups, a quarter as many identity experts beside them, and a token input of 256; and the
+    Vipalorn model of the same width, depth, heads and experts."""
+    W, L, H, D, V, rank, rot, E, top, ff, vocab = FAMILY_SIZES[size]
+    mlp = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": E, "top": top, "identity": E // 4,
+                                                              "groups": {"count": 4, "keep": 2}}}
+    space = {"type": "mamba2", "mixer": {"heads": 2 * W // 64, "vdim": 64, "state": 128, "groups": 8, "conv": 4,
+                                         "norm_groups": 8}}
+    attention = {"type": "attention", "mixer": {"heads": H, "kv_heads": H // 2, "dim": D, "vdim": V, "scale": D ** -0.5,
+                                                "rot": {"dims": D, "base": 500000.0, "scaling": {"factor": 8.0}},
+                                                "mask": {"size": 2048}, "softcap": 30.0}}
+    latent = {"type": "latent_attention", "mixer": {"heads": H, "dim": D, "rot_dim": rot, "vdim": V, "kv_rank": rank,
+                                                    "scale": (D + rot) ** -0.5, "rot": {"base": 10000.0, "dims": rot}}}
+    layers = [dict((space, attention, space, latent)[i % 4], mlp=mlp) for i in range(L)]
+    boz = {"architecture": "Bozasun", "vocab": vocab, "width": W, "layers": layers, "norm": {"eps": 1e-6},
+           "token_side": {"dim": 256}}
+    return boz, family_configs(size)[0]
+
+
 def run_family(args, names=("vipalorn", "qwen3"), configs=family_configs):
     """Prompt and decode throughput of a design at one size (random weights) beside the closest other model at
-    equal size (Vipalorn beside the dense Qwen3 decoder, Modasun beside Vipalorn, Mefatar beside Modasun), both through the generation
+    equal size (Vipalorn beside the dense Qwen3 decoder, Modasun beside Vipalorn, Mefatar beside Modasun, Bozasun beside Vipalorn), both through the generation
     loop: prompts of 512 and 2,048 tokens alone, and batches of 1, 8 and 32 sequences of 1,024 prompt tokens
     decoding `--steps` tokens each."""
     import torch
@@ -279,8 +302,8 @@ def main():
     ap.add_argument("--no-sweep", action="store_true", help="time the full context only, not 512 and the mean")
     ap.add_argument("--no-long", action="store_true",
                     help="skip the further sizes and lengths (contexts of 16 K and 32 K, batch 128 and 256, long prompts)")
-    ap.add_argument("--size", default="medium", choices=sorted(FAMILY_SIZES), help="layer sizes of --workload vipalorn, modasun and mefatar")
-    ap.add_argument("--workload", default="headline", choices=["headline", "qwen3-1.7b", "qwen3-32b", "vipalorn", "modasun", "mefatar"],
+    ap.add_argument("--size", default="medium", choices=sorted(FAMILY_SIZES), help="layer sizes of --workload vipalorn, modasun, mefatar and bozasun")
+    ap.add_argument("--workload", default="headline", choices=["headline", "qwen3-1.7b", "qwen3-32b", "vipalorn", "modasun", "mefatar", "bozasun"],
                     help="headline: BASELINE.json configs[2]; qwen3-*: configs[3] and configs[4]; vipalorn, modasun, mefatar: "
                          "that design at --size beside the closest other model at equal size")
     ap.add_argument("--prefill-tokens", type=int, default=2048, help="length of the prompt of the prefill figure")
@@ -308,6 +331,9 @@ def main():
         return 0
     if args.workload == "mefatar":
         print(json.dumps(run_family(args, names=("mefatar", "modasun"), configs=mefatar_configs)))
+        return 0
+    if args.workload == "bozasun":
+        print(json.dumps(run_family(args, names=("bozasun", "vipalorn"), configs=bozasun_configs)))
         return 0
     if args.workload != "headline":
         print(json.dumps(run_workload(args, 3 if args.workload == "qwen3-1.7b" else 4,

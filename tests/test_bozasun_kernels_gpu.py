@@ -94,7 +94,7 @@ def test_prepared_attention_over_chunks_with_capped_scores(nq, nkv, dim, vdim, r
     if chunk:
         _, other = attention_reference(proj[:, :C], bias[:C], qw, kw, rot, nq, nkv, dim, vdim, eps, scale, chunk + 1, softcap, dtype)
         assert float((other - out_ref).abs().max()) > 0.1 * float(out_ref.abs().max())
-    if softcap:
+    if softcap and softcap <= 30.0:
         _, other = attention_reference(proj[:, :C], bias[:C], qw, kw, rot, nq, nkv, dim, vdim, eps, scale, chunk, None, dtype)
         assert float((other - out_ref).abs().max()) > 0.02 * float(out_ref.abs().max())
     hd = head_size(dtype, dim, vdim)
