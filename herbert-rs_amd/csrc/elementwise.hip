@@ -1154,97 +1154,173 @@ extern "C" int hb_gate_heads(const void* attn, int dtype, const float* gate_rows
 // ------------------------------------------- a token's own input to the residual stream, layer by layer
 // With e = table[token, col0 .. col0 + D) (a token's row of a table, this layer's part of it):
 //     g = gelu_tanh(W_gate x) * e;   y = W_proj g;   x <- x + y / sqrt(mean(y^2) + eps) * w
-// x f32 [T, H] in place; W_gate [D, H], W_proj [H, D] and the table in one storage type; all arithmetic float32.
-// A workgroup takes TPB tokens: their rows of x lie in LDS, a wave takes gate rows in turn (a row of W_gate is
-// read once for all TPB tokens, the lanes share its columns), then a thread takes output columns (a row of
-// W_proj each), and the rows' sums of squares are added up by the block in a fixed order.
-template <class TW, int TPB>
+// x f32 [T, H] in place; W_gate [D, H], the table, and W_proj transposed [D, H] in one storage type; all arithmetic
+// float32. Three kernels, each of which fills the chip for a few tokens as for thousands:
+//   gate: a workgroup takes SIDE_TOKENS tokens and 4 x RW rows of W_gate; a wave takes RW of them, its lanes
+//     share a row's columns (whole lines of the matrix), every x is read once for the wave's RW rows; the sums
+//     over the lanes run in a fixed order; g f32 [T, D]; a step of few tokens gives a row to a whole workgroup;
+//   proj: a workgroup takes SIDE_TOKENS tokens (their g in LDS) and 64 columns of y; a lane takes a column,
+//     its weights W_proj^T [j, c] lie side by side for neighbouring lanes, the four waves a quarter of the
+//     gates each; y f32 [T, H];
+//   add: a workgroup a token: the row's mean of squares in a fixed order, then x += y / rms * w.
+#define SIDE_TOKENS 8
+template <class TW, int RW>
 __global__ void __launch_bounds__(256)
-token_side_kernel(float* __restrict__ x, const int* __restrict__ tokens, const TW* __restrict__ table, int table_ld,
-                  int col0, const TW* __restrict__ w_gate, const TW* __restrict__ w_proj,
-                  const float* __restrict__ norm_w, int T, int H, int D, float eps) {
-    extern __shared__ float side_lds[];            // [TPB][H] rows of x, then of y; [TPB][D] g
-    __shared__ float red[16];
-    float* const xs = side_lds;
-    float* const gs = side_lds + (size_t)TPB * H;
-    const int t0 = blockIdx.x * TPB, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int nt = T - t0 < TPB ? T - t0 : TPB;
-    for (int i = tid; i < TPB * H; i += 256) {
-        const int k = i / H;
-        xs[i] = k < nt ? x[(size_t)(t0 + k) * H + (i - k * H)] : 0.f;
+token_gate_kernel(const float* __restrict__ x, const int* __restrict__ tokens, const TW* __restrict__ table,
+                  int table_ld, int col0, const TW* __restrict__ w_gate, float* __restrict__ g, int T, int H, int D) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int t0 = blockIdx.y * SIDE_TOKENS;
+    const int j0 = (blockIdx.x * 4 + wave) * RW;
+    if (j0 >= D) return;
+    float acc[RW][SIDE_TOKENS];
+#pragma unroll
+    for (int r = 0; r < RW; ++r)
+#pragma unroll
+        for (int k = 0; k < SIDE_TOKENS; ++k) acc[r][k] = 0.f;
+    for (int c = lane; c < H; c += 64) {
+        float w[RW], xv[SIDE_TOKENS];
+#pragma unroll
+        for (int r = 0; r < RW; ++r) w[r] = j0 + r < D ? hb_to_float(w_gate[(size_t)(j0 + r) * H + c]) : 0.f;
+#pragma unroll
+        for (int k = 0; k < SIDE_TOKENS; ++k) xv[k] = t0 + k < T ? x[(size_t)(t0 + k) * H + c] : 0.f;
+#pragma unroll
+        for (int r = 0; r < RW; ++r)
+#pragma unroll
+            for (int k = 0; k < SIDE_TOKENS; ++k) acc[r][k] = fmaf(w[r], xv[k], acc[r][k]);
     }
-    __syncthreads();
-    for (int j = wave; j < D; j += 4) {
-        float acc[TPB];
 #pragma unroll
-        for (int k = 0; k < TPB; ++k) acc[k] = 0.f;
-        for (int c = lane; c < H; c += 64) {
-            const float w = hb_to_float(w_gate[(size_t)j * H + c]);
+    for (int r = 0; r < RW; ++r)
 #pragma unroll
-            for (int k = 0; k < TPB; ++k) acc[k] = fmaf(w, xs[k * H + c], acc[k]);
-        }
-#pragma unroll
-        for (int k = 0; k < TPB; ++k) {
-            const float z = hb_wave_sum(acc[k]);
-            if (lane == 0 && k < nt) {
+        for (int k = 0; k < SIDE_TOKENS; ++k) {
+            const float z = hb_wave_sum(acc[r][k]);
+            if (lane == 0 && j0 + r < D && t0 + k < T) {
                 const float gelu = 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
-                gs[k * D + j] = gelu * hb_to_float(table[(size_t)tokens[t0 + k] * table_ld + col0 + j]);
+                g[(size_t)(t0 + k) * D + j0 + r] = gelu * hb_to_float(table[(size_t)tokens[t0 + k] * table_ld + col0 + j0 + r]);
             }
         }
+}
+
+// (few tokens: all four waves of a workgroup share one row of W_gate, a quarter of its columns each)
+template <class TW>
+__global__ void __launch_bounds__(256)
+token_gate_few_kernel(const float* __restrict__ x, const int* __restrict__ tokens, const TW* __restrict__ table,
+                      int table_ld, int col0, const TW* __restrict__ w_gate, float* __restrict__ g, int T, int H, int D) {
+    __shared__ float part[4][SIDE_TOKENS];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int t0 = blockIdx.y * SIDE_TOKENS, j = blockIdx.x;
+    float acc[SIDE_TOKENS];
+#pragma unroll
+    for (int k = 0; k < SIDE_TOKENS; ++k) acc[k] = 0.f;
+#pragma unroll 4
+    for (int c = threadIdx.x; c < H; c += 256) {
+        const float w = hb_to_float(w_gate[(size_t)j * H + c]);
+#pragma unroll
+        for (int k = 0; k < SIDE_TOKENS; ++k) acc[k] = fmaf(w, t0 + k < T ? x[(size_t)(t0 + k) * H + c] : 0.f, acc[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < SIDE_TOKENS; ++k) {
+        const float z = hb_wave_sum(acc[k]);
+        if (lane == 0) part[wave][k] = z;
     }
     __syncthreads();
-    float ss[TPB];
-#pragma unroll
-    for (int k = 0; k < TPB; ++k) ss[k] = 0.f;
-    for (int c = tid; c < H; c += 256) {
-        float y[TPB];
-#pragma unroll
-        for (int k = 0; k < TPB; ++k) y[k] = 0.f;
-        for (int j = 0; j < D; ++j) {
-            const float w = hb_to_float(w_proj[(size_t)c * D + j]);
-#pragma unroll
-            for (int k = 0; k < TPB; ++k) y[k] = fmaf(w, gs[k * D + j], y[k]);
-        }
-#pragma unroll
-        for (int k = 0; k < TPB; ++k) {
-            xs[k * H + c] = y[k];                      // (this thread alone reads and writes column c from here on)
-            ss[k] = fmaf(y[k], y[k], ss[k]);
-        }
-    }
-#pragma unroll
-    for (int k = 0; k < TPB; ++k) ss[k] = hb_block_sum(ss[k], red);
-    for (int c = tid; c < H; c += 256) {
-        const float w = norm_w[c];
-#pragma unroll
-        for (int k = 0; k < TPB; ++k)
-            if (k < nt) x[(size_t)(t0 + k) * H + c] += xs[k * H + c] / sqrtf(ss[k] / (float)H + eps) * w;
+    const int k = threadIdx.x;
+    if (k < SIDE_TOKENS && t0 + k < T) {
+        const float z = ((part[0][k] + part[1][k]) + part[2][k]) + part[3][k];
+        const float gelu = 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+        g[(size_t)(t0 + k) * D + j] = gelu * hb_to_float(table[(size_t)tokens[t0 + k] * table_ld + col0 + j]);
     }
 }
 
+// (64 columns of y a workgroup; wave q takes the q-th quarter of the D gates, and the four partial sums of a
+// column are added in their order)
+template <class TW>
+__global__ void __launch_bounds__(256)
+token_proj_kernel(const float* __restrict__ g, const TW* __restrict__ w_proj_t, float* __restrict__ y, int T, int H,
+                  int D) {
+    extern __shared__ float side_g[];              // [SIDE_TOKENS][D], then the partial sums [3][SIDE_TOKENS][64]
+    float* const partial = side_g + SIDE_TOKENS * D;
+    const int t0 = blockIdx.y * SIDE_TOKENS;
+    const int lane = threadIdx.x & 63, q = threadIdx.x >> 6;
+    const int c = blockIdx.x * 64 + lane;
+    for (int i = threadIdx.x; i < SIDE_TOKENS * D; i += 256) {
+        const int k = i / D;
+        side_g[i] = t0 + k < T ? g[(size_t)(t0 + k) * D + (i - k * D)] : 0.f;
+    }
+    __syncthreads();
+    const int per = (D + 3) / 4;
+    const int j0 = q * per, j1 = j0 + per < D ? j0 + per : D;
+    float acc[SIDE_TOKENS];
+#pragma unroll
+    for (int k = 0; k < SIDE_TOKENS; ++k) acc[k] = 0.f;
+    if (c < H) {
+        // sixteen weights asked for at once (one after the other, each would wait for memory), then their products
+        for (int j = j0; j < j1; j += 16) {
+            float w[16];
+#pragma unroll
+            for (int o = 0; o < 16; ++o) w[o] = j + o < j1 ? hb_to_float(w_proj_t[(size_t)(j + o) * H + c]) : 0.f;
+#pragma unroll
+            for (int o = 0; o < 16; ++o) {
+                const int at = j + o < j1 ? j + o : j1 - 1;
+#pragma unroll
+                for (int k = 0; k < SIDE_TOKENS; ++k) acc[k] = fmaf(w[o], side_g[k * D + at], acc[k]);
+            }
+        }
+    }
+    if (q > 0) {
+#pragma unroll
+        for (int k = 0; k < SIDE_TOKENS; ++k) partial[((q - 1) * SIDE_TOKENS + k) * 64 + lane] = acc[k];
+    }
+    __syncthreads();
+    if (q > 0 || c >= H) return;
+#pragma unroll
+    for (int k = 0; k < SIDE_TOKENS; ++k) {
+        float sum = acc[k];
+#pragma unroll
+        for (int o = 0; o < 3; ++o) sum += partial[(o * SIDE_TOKENS + k) * 64 + lane];
+        if (t0 + k < T) y[(size_t)(t0 + k) * H + c] = sum;
+    }
+}
+
+__global__ void __launch_bounds__(256)
+add_normed_kernel(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ w, int H, float eps) {
+    __shared__ float red[16];
+    const size_t row = (size_t)blockIdx.x * H;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < H; c += 256) ss = fmaf(y[row + c], y[row + c], ss);
+    ss = hb_block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+    for (int c = threadIdx.x; c < H; c += 256) x[row + c] += y[row + c] * inv * w[c];
+}
+
+// g f32 [T, D] and y f32 [T, H] are the caller's scratch.
 extern "C" int hb_token_side(float* x, const int* tokens, const void* table, int table_ld, int col0, const void* w_gate,
-                             const void* w_proj, int dtype, const float* norm_w, int T, int H, int D, float eps,
-                             hipStream_t stream) {
+                             const void* w_proj_t, int dtype, const float* norm_w, float* g, float* y, int T, int H,
+                             int D, float eps, hipStream_t stream) {
     HB_REQUIRE(T > 0 && H > 0 && D > 0, "token input: empty input");
     HB_REQUIRE(col0 >= 0 && col0 + D <= table_ld, "token input: the layer's columns lie outside the table's rows");
-    const size_t per_token = ((size_t)H + D) * sizeof(float);
-    HB_REQUIRE(per_token <= 60 * 1024, "token input: a row of %d and %d gates do not fit the kernel's LDS", H, D);
-    const bool four = 4 * per_token <= 60 * 1024 && T >= 4;
-    const size_t lds = (four ? 4 : 1) * per_token;
+    const size_t lds = ((size_t)SIDE_TOKENS * D + 3 * SIDE_TOKENS * 64) * sizeof(float);
+    HB_REQUIRE(lds <= 60 * 1024, "token input: %d gates a token do not fit the kernel's LDS", D);
+    const int tiles = (T + SIDE_TOKENS - 1) / SIDE_TOKENS;
+    HB_REQUIRE(tiles <= 65535, "token input: too many tokens for the grid");
+    const bool many = T > 64;          // (few tokens: a row a workgroup, so that the gate's rows are spread over more waves)
+    HB_REQUIRE(D <= 65535, "token input: too many gates for the grid");
 #define HB_SIDE(TW)                                                                                                   \
     do {                                                                                                              \
-        if (four)                                                                                                     \
-            token_side_kernel<TW, 4><<<(T + 3) / 4, 256, lds, stream>>>(x, tokens, (const TW*)table, table_ld, col0,   \
-                                                                        (const TW*)w_gate, (const TW*)w_proj, norm_w, \
-                                                                        T, H, D, eps);                                \
+        if (many)                                                                                                     \
+            token_gate_kernel<TW, 4><<<dim3((D + 15) / 16, tiles), 256, 0, stream>>>(                                  \
+                x, tokens, (const TW*)table, table_ld, col0, (const TW*)w_gate, g, T, H, D);                          \
         else                                                                                                          \
-            token_side_kernel<TW, 1><<<T, 256, lds, stream>>>(x, tokens, (const TW*)table, table_ld, col0,            \
-                                                              (const TW*)w_gate, (const TW*)w_proj, norm_w, T, H, D,  \
-                                                              eps);                                                   \
+            token_gate_few_kernel<TW><<<dim3(D, tiles), 256, 0, stream>>>(                                             \
+                x, tokens, (const TW*)table, table_ld, col0, (const TW*)w_gate, g, T, H, D);                          \
+        HB_CHECK_LAUNCH("token_gate");                                                                                \
+        token_proj_kernel<TW><<<dim3((H + 63) / 64, tiles), 256, lds, stream>>>(g, (const TW*)w_proj_t, y, T, H, D);   \
+        HB_CHECK_LAUNCH("token_proj");                                                                                \
     } while (0)
     if (dtype == HB_F32) HB_SIDE(float);
     else if (dtype == HB_BF16) HB_SIDE(bf16);
     else HB_REQUIRE(false, "token input: unknown dtype %d", dtype);
 #undef HB_SIDE
-    HB_CHECK_LAUNCH("token_side");
+    add_normed_kernel<<<T, 256, 0, stream>>>(x, y, norm_w, H, eps);
+    HB_CHECK_LAUNCH("token_add_normed");
     return 0;
 }

@@ -659,9 +659,10 @@ extern "C" int hb_channel_decay(const float* z, int ld, const float* A_log, cons
 // left); dt_pre: column dt_off + h of proj's rows (f32, ld apart); state f32 [slots, heads, N, P]; y f32
 // [T, heads x P]. Everything is float32.
 // A workgroup is one wave on (16 columns of S, head, sequence): a column's N numbers lie over 4 lanes, lane j
-// holding rows j, j + 4, ... (NR of them), so the sum over N is NR products a lane and two exchanges, in one
-// order whatever the step holds. The tokens are a chain; their inputs come through LDS eight tokens at a time,
-// so that the chain waits for memory once in eight steps.
+// holding rows j NR .. (j + 1) NR - 1, so the sum over N is NR products a lane and two exchanges, in one order
+// whatever the step holds. The tokens are a chain; their inputs come through LDS eight tokens at a time, and the
+// next eight are asked for (into registers, every load of a lane at once, no branch between them) before the
+// eight at hand are walked, so the chain does not wait for memory.
 #define SSM_COLS 16
 #define SSM_TOKENS 8
 template <int NR>
@@ -670,7 +671,11 @@ ssm_scan_kernel(const float* __restrict__ u, int ldu, const float* __restrict__ 
                 const float* __restrict__ dt_bias, const float* __restrict__ A_log, const float* __restrict__ Dskip,
                 float* __restrict__ state, const int* __restrict__ seq_starts, const int* __restrict__ slots,
                 float* __restrict__ y, int heads, int groups, int N, int P) {
-    extern __shared__ float ssm_lds[];     // [SSM_TOKENS][B: N | C: N | x: SSM_COLS | dt, a]
+    constexpr int MAXN = 4 * NR;                        // rows that the lanes' registers hold (those from N on stay zero)
+    constexpr int ROW = 2 * MAXN + SSM_COLS;            // a token's inputs: B | C | x
+    constexpr int STRIDE = ROW + 4;                     // then dt, the decay, and two unused
+    constexpr int PER = (SSM_TOKENS * ROW + HB_WAVE - 1) / HB_WAVE;
+    __shared__ __attribute__((aligned(16))) float in_lds[SSM_TOKENS * STRIDE];
     const int tile = blockIdx.x, h = blockIdx.y, seq = blockIdx.z;
     const int lane = threadIdx.x, col = lane >> 2, part = lane & 3;
     const int p = tile * SSM_COLS + col;
@@ -678,47 +683,72 @@ ssm_scan_kernel(const float* __restrict__ u, int ldu, const float* __restrict__ 
     const int g = h / (heads / groups);
     const int first = seq_starts[seq], n_tok = seq_starts[seq + 1] - first;
     const int inner = heads * P;
-    const int stride = 2 * N + SSM_COLS + 2;
     float* S = state + (((size_t)slots[seq] * heads + h) * N) * P;
     float s[NR];
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
-        const int n = part + 4 * i;
+        const int n = part * NR + i;
         s[i] = (live && n < N) ? S[(size_t)n * P + p] : 0.f;
     }
     const float rate = expf(A_log[h]), bias = dt_bias[h], skip = Dskip[h];
+    // where this lane's PER numbers of a chunk lie in a token's row of u (below zero: nowhere; they are zeros)
+    int src[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int idx = lane + HB_WAVE * i;
+        const int e = idx % ROW;
+        int off = -1;
+        if (idx < SSM_TOKENS * ROW) {
+            if (e < MAXN) off = e < N ? inner + g * N + e : -1;
+            else if (e < 2 * MAXN) off = e - MAXN < N ? inner + (groups + g) * N + (e - MAXN) : -1;
+            else off = tile * SSM_COLS + (e - 2 * MAXN) < P ? h * P + tile * SSM_COLS + (e - 2 * MAXN) : -1;
+        }
+        src[i] = off;
+    }
+    float pre[PER], pre_dt = 0.f;
+    auto fetch = [&](int t0) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int k = (lane + HB_WAVE * i) / ROW;
+            const bool in = src[i] >= 0 && t0 + k < n_tok;
+            pre[i] = in ? u[(size_t)(first + t0 + k) * ldu + src[i]] : 0.f;
+        }
+        pre_dt = (lane < SSM_TOKENS && t0 + lane < n_tok) ? proj[(size_t)(first + t0 + lane) * ld + dt_off + h] : 0.f;
+    };
+    fetch(0);
     for (int t0 = 0; t0 < n_tok; t0 += SSM_TOKENS) {
         const int nt = n_tok - t0 < SSM_TOKENS ? n_tok - t0 : SSM_TOKENS;
-        __syncthreads();
-        for (int idx = lane; idx < nt * stride; idx += HB_WAVE) {
-            const int k = idx / stride, e = idx - k * stride;
-            const size_t row = (size_t)(first + t0 + k);
-            float v;
-            if (e < 2 * N) {
-                v = u[row * ldu + inner + (e < N ? g * N + e : (groups + g) * N + (e - N))];
-            } else if (e < 2 * N + SSM_COLS) {
-                const int pc = tile * SSM_COLS + (e - 2 * N);
-                v = pc < P ? u[row * ldu + h * P + pc] : 0.f;
-            } else {
-                const float z = proj[row * ld + dt_off + h] + bias;
-                const float dt = z > 20.f ? z : log1pf(expf(z));
-                v = e == 2 * N + SSM_COLS ? dt : expf(-rate * dt);
-            }
-            ssm_lds[idx] = v;
+        __syncthreads();                 // (the chunk before has been walked)
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int idx = lane + HB_WAVE * i;
+            if (idx < SSM_TOKENS * ROW) in_lds[(idx / ROW) * STRIDE + idx % ROW] = pre[i];
+        }
+        if (lane < SSM_TOKENS) {
+            const float z = pre_dt + bias;
+            const float dt = z > 20.f ? z : log1pf(expf(z));
+            in_lds[lane * STRIDE + ROW] = dt;
+            in_lds[lane * STRIDE + ROW + 1] = expf(-rate * dt);
         }
         __syncthreads();
+        if (t0 + SSM_TOKENS < n_tok) fetch(t0 + SSM_TOKENS);
         for (int k = 0; k < nt; ++k) {
-            const float* in = ssm_lds + k * stride;
-            const float x = in[2 * N + col], dt = in[2 * N + SSM_COLS], a = in[2 * N + SSM_COLS + 1];
+            const float* in = in_lds + k * STRIDE;
+            const float x = in[2 * MAXN + col], dt = in[ROW], a = in[ROW + 1];
             const float dx = dt * x;
             float acc = 0.f;
 #pragma unroll
-            for (int i = 0; i < NR; ++i) {
-                const int n = part + 4 * i;
-                if (n < N) {
-                    s[i] = fmaf(a, s[i], dx * in[n]);
-                    acc = fmaf(s[i], in[N + n], acc);
-                }
+            for (int i = 0; i < NR; i += 4) {
+                const float4 b = *(const float4*)(in + part * NR + i);
+                const float4 c = *(const float4*)(in + MAXN + part * NR + i);
+                s[i] = fmaf(a, s[i], dx * b.x);
+                s[i + 1] = fmaf(a, s[i + 1], dx * b.y);
+                s[i + 2] = fmaf(a, s[i + 2], dx * b.z);
+                s[i + 3] = fmaf(a, s[i + 3], dx * b.w);
+                acc = fmaf(s[i], c.x, acc);
+                acc = fmaf(s[i + 1], c.y, acc);
+                acc = fmaf(s[i + 2], c.z, acc);
+                acc = fmaf(s[i + 3], c.w, acc);
             }
             acc += __shfl_xor(acc, 1, HB_WAVE);
             acc += __shfl_xor(acc, 2, HB_WAVE);
@@ -727,7 +757,7 @@ ssm_scan_kernel(const float* __restrict__ u, int ldu, const float* __restrict__ 
     }
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
-        const int n = part + 4 * i;
+        const int n = part * NR + i;
         if (live && n < N) S[(size_t)n * P + p] = s[i];
     }
 }
@@ -743,8 +773,7 @@ extern "C" int hb_ssm_scan(const float* u, int ldu, const float* proj, int ld, i
                "state-space walk: the columns lie outside their rows");
     HB_REQUIRE(heads <= 65535 && B <= 65535, "state-space walk: too many heads or sequences for the grid");
     const dim3 grid((P + SSM_COLS - 1) / SSM_COLS, heads, B);
-    const size_t lds = (size_t)SSM_TOKENS * (2 * N + SSM_COLS + 2) * sizeof(float);
-#define HB_SSM(NRV) ssm_scan_kernel<NRV><<<grid, HB_WAVE, lds, stream>>>(u, ldu, proj, ld, dt_off, dt_bias, A_log, Dskip, \
+#define HB_SSM(NRV) ssm_scan_kernel<NRV><<<grid, HB_WAVE, 0, stream>>>(u, ldu, proj, ld, dt_off, dt_bias, A_log, Dskip, \
                                                                          state, seq_starts, slots, y, heads, groups, N, P)
     if (N <= 16) HB_SSM(4);
     else if (N <= 32) HB_SSM(8);

@@ -579,22 +579,25 @@ def add_bias(x, bias):
     lib.call("elementwise", "hb_add_bias", x.data_ptr(), bias.data_ptr(), T, H, _stream())
 
 
-def token_side(x, token_ids, table, col0, w_gate, w_proj, norm_w, eps):
+def token_side(x, token_ids, table, col0, w_gate, w_proj_t, norm_w, eps, g, y):
     """x += rmsnorm(W_proj (gelu_tanh(W_gate x) * table[token, col0 : col0 + D])) * norm_w, row by row and in
-    place: x f32 [T, H], token_ids int32 [T], table [V, ld], W_gate [D, H], W_proj [H, D] (one dtype), norm_w f32 [H]."""
+    place: x f32 [T, H], token_ids int32 [T], table [V, ld], W_gate [D, H], W_proj transposed [D, H] (one dtype),
+    norm_w f32 [H]; g f32 [T, D] and y f32 [T, H] are scratch."""
     T, H = x.shape
     D = w_gate.shape[0]
     _check(x, "x", torch.float32, (T, H))
     _check(token_ids, "token_ids", torch.int32, (T,))
     _check(table, "table", w_gate.dtype, (None, None))
     _check(w_gate, "gate", None, (D, H))
-    _check(w_proj, "proj", w_gate.dtype, (H, D))
+    _check(w_proj_t, "proj (transposed)", w_gate.dtype, (D, H))
     _check(norm_w, "norm", torch.float32, (H,))
+    _check(g, "g", torch.float32, (T, D))
+    _check(y, "y", torch.float32, (T, H))
     if col0 < 0 or col0 + D > table.shape[1]:
         raise BackendError("token input: the layer's columns lie outside the table's rows")
     lib.call("elementwise", "hb_token_side", x.data_ptr(), token_ids.data_ptr(), table.data_ptr(), table.shape[1],
-             int(col0), w_gate.data_ptr(), w_proj.data_ptr(), dtype_code(w_gate), norm_w.data_ptr(), T, H, D, float(eps),
-             _stream())
+             int(col0), w_gate.data_ptr(), w_proj_t.data_ptr(), dtype_code(w_gate), norm_w.data_ptr(), g.data_ptr(),
+             y.data_ptr(), T, H, D, float(eps), _stream())
 
 
 def gate_heads(attn, gate_rows, g_off, out, nq, hd, vdim):

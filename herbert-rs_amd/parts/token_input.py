@@ -5,10 +5,13 @@ e = that token's row for this layer (columns [i dim, (i + 1) dim) of the table):
 
     g = gelu_tanh(W_gate x) * e;   y = W_proj g;   x <- x + y / sqrt(mean(y^2) + eps) * w
 
-The gate reads the residual stream x itself, not a normed copy of it. One kernel does all of it, in float32
-arithmetic in either mode (the matrices and the table are kept in the compute dtype). The table is one tensor
-for all layers and is kept on the GPU once.
+The gate reads the residual stream x itself, not a normed copy of it. Three small kernels do it (the gate, the
+second product, the norm with the sum), in float32 arithmetic in either mode; the matrices and the table are kept in
+the compute dtype, W_proj transposed so that neighbouring threads read neighbouring weights. The table is one
+tensor for all layers and is kept on the GPU once.
 """
+import torch
+
 from ..kernels import ops
 from ..weights import TensorNeed
 from .base import Part
@@ -26,7 +29,7 @@ class GatedTableInput(Part):
         if not 0 <= self.layer < self.layers or self.dim <= 0:
             raise ValueError(f"part {self.layer} of a table of {self.layers} parts of {self.dim}")
         self.names = dict(names)
-        self.table = self.gate = self.proj = self.norm_w = None
+        self.table = self.gate = self.proj_t = self.norm_w = None
 
     def tensor_needs(self):
         n = self.names
@@ -38,9 +41,12 @@ class GatedTableInput(Part):
     def load(self, tensors, rt):
         n = self.names
         self.table = rt.shared_weight(n["table"], tensors[n["table"]])
-        self.gate, self.proj = rt.weight(tensors[n["gate"]]), rt.weight(tensors[n["proj"]])
+        self.gate, self.proj_t = rt.weight(tensors[n["gate"]]), rt.weight(tensors[n["proj"]]).t().contiguous()
         self.norm_w = rt.weight(tensors[n["norm"]], matrix=False)
 
     def forward(self, ctx, x):
-        ops.token_side(x, ctx.meta.token_ids, self.table, self.layer * self.dim, self.gate, self.proj, self.norm_w,
-                       self.eps)
+        T = x.shape[0]
+        g = ctx.rt.buffer("token_input_gates", (T, self.dim), torch.float32)
+        y = ctx.rt.buffer("token_input_rows", (T, self.hidden_size), torch.float32)
+        ops.token_side(x, ctx.meta.token_ids, self.table, self.layer * self.dim, self.gate, self.proj_t, self.norm_w,
+                       self.eps, g, y)

@@ -274,5 +274,6 @@ def test_token_input(T, H, D, layers, layer):
         tb, gt, pj = table.to(dtype), gate.to(dtype), proj.to(dtype)
         want = plain.token_side(x, tb.float()[tokens][:, layer * D:(layer + 1) * D], {"gate": gt.float(), "proj": pj.float(), "norm": norm_w}, 1e-5)
         xg = x.to(DEV).clone()
-        ops.token_side(xg, tokens.to(torch.int32).to(DEV), g(tb), layer * D, g(gt), g(pj), g(norm_w), 1e-5)
+        ops.token_side(xg, tokens.to(torch.int32).to(DEV), g(tb), layer * D, g(gt), g(pj.t()), g(norm_w), 1e-5,
+                       torch.empty(T, D, device=DEV), torch.empty(T, H, device=DEV))
         assert float((xg.cpu() - want).abs().max()) <= tol * float(want.abs().max())
