@@ -1180,9 +1180,11 @@ token_gate_kernel(const float* __restrict__ x, const int* __restrict__ tokens, c
     for (int c = lane; c < H; c += 64) {
         float w[RW], xv[SIDE_TOKENS];
 #pragma unroll
-        for (int r = 0; r < RW; ++r) w[r] = j0 + r < D ? hb_to_float(w_gate[(size_t)(j0 + r) * H + c]) : 0.f;
+        // (rows past the end read the last row again: a load under a condition would wait for the one before it,
+        //  and what is summed for such a row is never stored)
+        for (int r = 0; r < RW; ++r) w[r] = hb_to_float(w_gate[(size_t)(j0 + r < D ? j0 + r : D - 1) * H + c]);
 #pragma unroll
-        for (int k = 0; k < SIDE_TOKENS; ++k) xv[k] = t0 + k < T ? x[(size_t)(t0 + k) * H + c] : 0.f;
+        for (int k = 0; k < SIDE_TOKENS; ++k) xv[k] = x[(size_t)(t0 + k < T ? t0 + k : T - 1) * H + c];
 #pragma unroll
         for (int r = 0; r < RW; ++r)
 #pragma unroll
@@ -1215,7 +1217,7 @@ token_gate_few_kernel(const float* __restrict__ x, const int* __restrict__ token
     for (int c = threadIdx.x; c < H; c += 256) {
         const float w = hb_to_float(w_gate[(size_t)j * H + c]);
 #pragma unroll
-        for (int k = 0; k < SIDE_TOKENS; ++k) acc[k] = fmaf(w, t0 + k < T ? x[(size_t)(t0 + k) * H + c] : 0.f, acc[k]);
+        for (int k = 0; k < SIDE_TOKENS; ++k) acc[k] = fmaf(w, x[(size_t)(t0 + k < T ? t0 + k : T - 1) * H + c], acc[k]);
     }
 #pragma unroll
     for (int k = 0; k < SIDE_TOKENS; ++k) {
@@ -1257,12 +1259,15 @@ token_proj_kernel(const float* __restrict__ g, const TW* __restrict__ w_proj_t, 
         for (int j = j0; j < j1; j += 16) {
             float w[16];
 #pragma unroll
-            for (int o = 0; o < 16; ++o) w[o] = j + o < j1 ? hb_to_float(w_proj_t[(size_t)(j + o) * H + c]) : 0.f;
+            // (no load stands under a condition, which would make it wait for the one before: past the end the last
+            //  weight is read again and counts as zero)
+            for (int o = 0; o < 16; ++o) w[o] = hb_to_float(w_proj_t[(size_t)(j + o < j1 ? j + o : j1 - 1) * H + c]);
 #pragma unroll
             for (int o = 0; o < 16; ++o) {
                 const int at = j + o < j1 ? j + o : j1 - 1;
+                const float wo = j + o < j1 ? w[o] : 0.f;
 #pragma unroll
-                for (int k = 0; k < SIDE_TOKENS; ++k) acc[k] = fmaf(w[o], side_g[k * D + at], acc[k]);
+                for (int k = 0; k < SIDE_TOKENS; ++k) acc[k] = fmaf(wo, side_g[k * D + at], acc[k]);
             }
         }
     }

@@ -658,27 +658,28 @@ extern "C" int hb_channel_decay(const float* z, int ld, const float* A_log, cons
 // u f32 [T, ldu]: a row's columns are [x: heads x P | B: groups x N | C: groups x N] (what the convolution
 // left); dt_pre: column dt_off + h of proj's rows (f32, ld apart); state f32 [slots, heads, N, P]; y f32
 // [T, heads x P]. Everything is float32.
-// A workgroup is one wave on (16 columns of S, head, sequence): a column's N numbers lie over 4 lanes, lane j
-// holding rows j NR .. (j + 1) NR - 1, so the sum over N is NR products a lane and two exchanges, in one order
-// whatever the step holds. The tokens are a chain; their inputs come through LDS eight tokens at a time, and the
-// next eight are asked for (into registers, every load of a lane at once, no branch between them) before the
-// eight at hand are walked, so the chain does not wait for memory.
-#define SSM_COLS 16
+// A workgroup is four waves on (256 / LPC columns of S, head, sequence): a column's N numbers lie over LPC lanes
+// (4, 8 or 16), lane j holding rows j NR .. (j + 1) NR - 1, so the sum over N is NR products a lane and a few
+// exchanges, in one order whatever the step holds; the more lanes a column has, the more waves a step of one
+// sequence has and the shorter each wave's chain of work a token. The tokens are a chain; their inputs come
+// through LDS eight tokens at a time, loaded by all four waves together, and the next eight are asked for (into
+// registers) before the eight at hand are walked, so the chain does not wait for memory.
 #define SSM_TOKENS 8
-template <int NR>
-__global__ void __launch_bounds__(HB_WAVE)
+template <int NR, int LPC>
+__global__ void __launch_bounds__(256)
 ssm_scan_kernel(const float* __restrict__ u, int ldu, const float* __restrict__ proj, int ld, int dt_off,
                 const float* __restrict__ dt_bias, const float* __restrict__ A_log, const float* __restrict__ Dskip,
                 float* __restrict__ state, const int* __restrict__ seq_starts, const int* __restrict__ slots,
                 float* __restrict__ y, int heads, int groups, int N, int P) {
-    constexpr int MAXN = 4 * NR;                        // rows that the lanes' registers hold (those from N on stay zero)
-    constexpr int ROW = 2 * MAXN + SSM_COLS;            // a token's inputs: B | C | x
+    constexpr int CPW = 256 / LPC;                      // columns a workgroup
+    constexpr int MAXN = LPC * NR;                      // rows that the lanes' registers hold (those from N on stay zero)
+    constexpr int ROW = 2 * MAXN + CPW;                 // a token's inputs: B | C | x
     constexpr int STRIDE = ROW + 4;                     // then dt, the decay, and two unused
-    constexpr int PER = (SSM_TOKENS * ROW + HB_WAVE - 1) / HB_WAVE;
+    constexpr int PER = (SSM_TOKENS * ROW + 255) / 256;
     __shared__ __attribute__((aligned(16))) float in_lds[SSM_TOKENS * STRIDE];
     const int tile = blockIdx.x, h = blockIdx.y, seq = blockIdx.z;
-    const int lane = threadIdx.x, col = lane >> 2, part = lane & 3;
-    const int p = tile * SSM_COLS + col;
+    const int tid = threadIdx.x, col = tid / LPC, part = tid % LPC;
+    const int p = tile * CPW + col;
     const bool live = p < P;
     const int g = h / (heads / groups);
     const int first = seq_starts[seq], n_tok = seq_starts[seq + 1] - first;
@@ -688,20 +689,21 @@ ssm_scan_kernel(const float* __restrict__ u, int ldu, const float* __restrict__ 
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
         const int n = part * NR + i;
-        s[i] = (live && n < N) ? S[(size_t)n * P + p] : 0.f;
+        const float held = S[(size_t)(n < N ? n : N - 1) * P + (live ? p : P - 1)];
+        s[i] = (live && n < N) ? held : 0.f;
     }
     const float rate = expf(A_log[h]), bias = dt_bias[h], skip = Dskip[h];
-    // where this lane's PER numbers of a chunk lie in a token's row of u (below zero: nowhere; they are zeros)
+    // where this thread's PER numbers of a chunk lie in a token's row of u (below zero: nowhere; they are zeros)
     int src[PER];
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
-        const int idx = lane + HB_WAVE * i;
+        const int idx = tid + 256 * i;
         const int e = idx % ROW;
         int off = -1;
         if (idx < SSM_TOKENS * ROW) {
             if (e < MAXN) off = e < N ? inner + g * N + e : -1;
             else if (e < 2 * MAXN) off = e - MAXN < N ? inner + (groups + g) * N + (e - MAXN) : -1;
-            else off = tile * SSM_COLS + (e - 2 * MAXN) < P ? h * P + tile * SSM_COLS + (e - 2 * MAXN) : -1;
+            else off = tile * CPW + (e - 2 * MAXN) < P ? h * P + tile * CPW + (e - 2 * MAXN) : -1;
         }
         src[i] = off;
     }
@@ -709,11 +711,10 @@ ssm_scan_kernel(const float* __restrict__ u, int ldu, const float* __restrict__ 
     auto fetch = [&](int t0) {
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
-            const int k = (lane + HB_WAVE * i) / ROW;
-            const bool in = src[i] >= 0 && t0 + k < n_tok;
-            pre[i] = in ? u[(size_t)(first + t0 + k) * ldu + src[i]] : 0.f;
+            const int k = (tid + 256 * i) / ROW;
+            pre[i] = (src[i] >= 0 && t0 + k < n_tok) ? u[(size_t)(first + t0 + k) * ldu + src[i]] : 0.f;
         }
-        pre_dt = (lane < SSM_TOKENS && t0 + lane < n_tok) ? proj[(size_t)(first + t0 + lane) * ld + dt_off + h] : 0.f;
+        pre_dt = (tid < SSM_TOKENS && t0 + tid < n_tok) ? proj[(size_t)(first + t0 + tid) * ld + dt_off + h] : 0.f;
     };
     fetch(0);
     for (int t0 = 0; t0 < n_tok; t0 += SSM_TOKENS) {
@@ -721,14 +722,14 @@ ssm_scan_kernel(const float* __restrict__ u, int ldu, const float* __restrict__ 
         __syncthreads();                 // (the chunk before has been walked)
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
-            const int idx = lane + HB_WAVE * i;
+            const int idx = tid + 256 * i;
             if (idx < SSM_TOKENS * ROW) in_lds[(idx / ROW) * STRIDE + idx % ROW] = pre[i];
         }
-        if (lane < SSM_TOKENS) {
+        if (tid < SSM_TOKENS) {
             const float z = pre_dt + bias;
             const float dt = z > 20.f ? z : log1pf(expf(z));
-            in_lds[lane * STRIDE + ROW] = dt;
-            in_lds[lane * STRIDE + ROW + 1] = expf(-rate * dt);
+            in_lds[tid * STRIDE + ROW] = dt;
+            in_lds[tid * STRIDE + ROW + 1] = expf(-rate * dt);
         }
         __syncthreads();
         if (t0 + SSM_TOKENS < n_tok) fetch(t0 + SSM_TOKENS);
@@ -750,8 +751,8 @@ ssm_scan_kernel(const float* __restrict__ u, int ldu, const float* __restrict__ 
                 acc = fmaf(s[i + 2], c.z, acc);
                 acc = fmaf(s[i + 3], c.w, acc);
             }
-            acc += __shfl_xor(acc, 1, HB_WAVE);
-            acc += __shfl_xor(acc, 2, HB_WAVE);
+#pragma unroll
+            for (int off = 1; off < LPC; off <<= 1) acc += __shfl_xor(acc, off, HB_WAVE);
             if (live && part == 0) y[(size_t)(first + t0 + k) * inner + h * P + p] = fmaf(skip, x, acc);
         }
     }
@@ -772,14 +773,14 @@ extern "C" int hb_ssm_scan(const float* u, int ldu, const float* proj, int ld, i
     HB_REQUIRE(ldu >= heads * P + 2 * groups * N && dt_off >= 0 && dt_off + heads <= ld,
                "state-space walk: the columns lie outside their rows");
     HB_REQUIRE(heads <= 65535 && B <= 65535, "state-space walk: too many heads or sequences for the grid");
-    const dim3 grid((P + SSM_COLS - 1) / SSM_COLS, heads, B);
-#define HB_SSM(NRV) ssm_scan_kernel<NRV><<<grid, HB_WAVE, 0, stream>>>(u, ldu, proj, ld, dt_off, dt_bias, A_log, Dskip, \
-                                                                         state, seq_starts, slots, y, heads, groups, N, P)
-    if (N <= 16) HB_SSM(4);
-    else if (N <= 32) HB_SSM(8);
-    else if (N <= 64) HB_SSM(16);
-    else if (N <= 128) HB_SSM(32);
-    else HB_SSM(64);
+#define HB_SSM(NRV, LPCV)                                                                                              \
+    ssm_scan_kernel<NRV, LPCV><<<dim3((P + 256 / LPCV - 1) / (256 / LPCV), heads, B), 256, 0, stream>>>(               \
+        u, ldu, proj, ld, dt_off, dt_bias, A_log, Dskip, state, seq_starts, slots, y, heads, groups, N, P)
+    if (N <= 16) HB_SSM(4, 4);
+    else if (N <= 32) HB_SSM(4, 8);
+    else if (N <= 64) HB_SSM(4, 16);
+    else if (N <= 128) HB_SSM(8, 16);
+    else HB_SSM(16, 16);
 #undef HB_SSM
     HB_CHECK_LAUNCH("ssm_scan");
     return 0;
