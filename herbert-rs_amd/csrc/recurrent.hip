@@ -656,8 +656,10 @@ extern "C" int hb_channel_decay(const float* z, int ld, const float* A_log, cons
 // every token, with dt = softplus(dt_pre[h] + dt_bias[h]) and a = exp(-exp(A_log[h]) dt):
 //     S <- a S + dt B x^T;   y = S^T C + D[h] x.
 // u f32 [T, ldu]: a row's columns are [x: heads x P | B: groups x N | C: groups x N] (what the convolution
-// left); dt_pre: column dt_off + h of proj's rows (f32, ld apart); state f32 [slots, heads, N, P]; y f32
-// [T, heads x P]. Everything is float32.
+// left); dt_pre: column dt_off + h of proj's rows (f32, ld apart); y f32 [T, heads x P]. Everything is float32.
+// The state is the kernel's own: f32 [slots, heads, tiles, 256, NR], every thread's NR numbers of a (slot, head,
+// tile of columns) side by side, so that a step of single tokens streams it in and out in whole lines; rows
+// from N on and columns from P on are zeros and stay zeros.
 // A workgroup is four waves on (256 / LPC columns of S, head, sequence): a column's N numbers lie over LPC lanes
 // (4, 8 or 16), lane j holding rows j NR .. (j + 1) NR - 1, so the sum over N is NR products a lane and a few
 // exchanges, in one order whatever the step holds; the more lanes a column has, the more waves a step of one
@@ -684,13 +686,12 @@ ssm_scan_kernel(const float* __restrict__ u, int ldu, const float* __restrict__ 
     const int g = h / (heads / groups);
     const int first = seq_starts[seq], n_tok = seq_starts[seq + 1] - first;
     const int inner = heads * P;
-    float* S = state + (((size_t)slots[seq] * heads + h) * N) * P;
+    float* S = state + ((((size_t)slots[seq] * heads + h) * gridDim.x + tile) * 256 + tid) * NR;
     float s[NR];
 #pragma unroll
-    for (int i = 0; i < NR; ++i) {
-        const int n = part * NR + i;
-        const float held = S[(size_t)(n < N ? n : N - 1) * P + (live ? p : P - 1)];
-        s[i] = (live && n < N) ? held : 0.f;
+    for (int i = 0; i < NR; i += 4) {
+        const float4 held = *(const float4*)(S + i);
+        s[i] = held.x, s[i + 1] = held.y, s[i + 2] = held.z, s[i + 3] = held.w;
     }
     const float rate = expf(A_log[h]), bias = dt_bias[h], skip = Dskip[h];
     // where this thread's PER numbers of a chunk lie in a token's row of u (below zero: nowhere; they are zeros)
@@ -757,17 +758,33 @@ ssm_scan_kernel(const float* __restrict__ u, int ldu, const float* __restrict__ 
         }
     }
 #pragma unroll
-    for (int i = 0; i < NR; ++i) {
-        const int n = part * NR + i;
-        if (live && n < N) S[(size_t)n * P + p] = s[i];
-    }
+    for (int i = 0; i < NR; i += 4) *(float4*)(S + i) = make_float4(s[i], s[i + 1], s[i + 2], s[i + 3]);
+}
+
+// How the kernel lays a head's state out: rows a lane (NR), lanes a column (LPC); 256 / LPC columns a tile.
+static void ssm_layout(int N, int* nr, int* lpc) {
+    if (N <= 16) *nr = 4, *lpc = 4;
+    else if (N <= 32) *nr = 4, *lpc = 8;
+    else if (N <= 64) *nr = 4, *lpc = 16;
+    else if (N <= 128) *nr = 8, *lpc = 16;
+    else *nr = 16, *lpc = 16;
+}
+
+// floats of state a (slot, head) for a state of N rows and P columns
+extern "C" int hb_ssm_state_floats(int N, int P) {
+    int nr, lpc;
+    ssm_layout(N, &nr, &lpc);
+    const int cpw = 256 / lpc;
+    return (P + cpw - 1) / cpw * 256 * nr;
 }
 
 extern "C" int hb_ssm_scan(const float* u, int ldu, const float* proj, int ld, int dt_off, const float* dt_bias,
                            const float* A_log, const float* Dskip, float* state, const int* seq_starts,
                            const int* slots, float* y, int B, int heads, int groups, int N, int P,
-                           hipStream_t stream) {
+                           int state_floats, hipStream_t stream) {
     HB_REQUIRE(B > 0 && heads > 0 && groups > 0 && N > 0 && P > 0, "state-space walk: empty input");
+    HB_REQUIRE(N <= 256 && state_floats == hb_ssm_state_floats(N, P),
+               "state-space walk: a head's state of %d floats is not the kernel's layout for %d x %d", state_floats, N, P);
     HB_REQUIRE(heads % groups == 0, "state-space walk: %d heads in %d groups", heads, groups);
     HB_REQUIRE(N <= 256, "state-space walk: a state of %d rows, the kernel takes up to 256", N);
     HB_REQUIRE(ldu >= heads * P + 2 * groups * N && dt_off >= 0 && dt_off + heads <= ld,
@@ -776,10 +793,12 @@ extern "C" int hb_ssm_scan(const float* u, int ldu, const float* proj, int ld, i
 #define HB_SSM(NRV, LPCV)                                                                                              \
     ssm_scan_kernel<NRV, LPCV><<<dim3((P + 256 / LPCV - 1) / (256 / LPCV), heads, B), 256, 0, stream>>>(               \
         u, ldu, proj, ld, dt_off, dt_bias, A_log, Dskip, state, seq_starts, slots, y, heads, groups, N, P)
-    if (N <= 16) HB_SSM(4, 4);
-    else if (N <= 32) HB_SSM(4, 8);
-    else if (N <= 64) HB_SSM(4, 16);
-    else if (N <= 128) HB_SSM(8, 16);
+    int nr, lpc;
+    ssm_layout(N, &nr, &lpc);
+    if (nr == 4 && lpc == 4) HB_SSM(4, 4);
+    else if (nr == 4 && lpc == 8) HB_SSM(4, 8);
+    else if (nr == 4) HB_SSM(4, 16);
+    else if (nr == 8) HB_SSM(8, 16);
     else HB_SSM(16, 16);
 #undef HB_SSM
     HB_CHECK_LAUNCH("ssm_scan");

@@ -45,7 +45,7 @@ SIGNATURES = {
     },
     "recurrent": {
         "hb_conv_silu": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _I, _P, _P],
-        "hb_ssm_scan": [_P, _I, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+        "hb_ssm_scan": [_P, _I, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
         "hb_gated_group_norm": [_P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _P],
         "hb_gated_delta": [_P, _I, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
         "hb_filter_state": [_P, _I, _P, _P, _P, _I, _I, _I, _P, _P],

@@ -41,17 +41,28 @@ def conv_silu(proj, taps, conv_state, meta, out, n_unit, unit_dim, n_scaled, sca
 MAX_SSM_STATE = 256
 
 
+def ssm_state_floats(N, P):
+    """Floats of state that the walk's kernel keeps for a head of N rows and P columns (its own layout: every
+    thread's numbers side by side, rows and columns rounded up to what its lanes hold). The kernel's entry point
+    refuses a state of another size, so the two cannot drift apart unseen."""
+    if not 0 < N <= MAX_SSM_STATE or P <= 0:
+        raise BackendError(f"state-space walk: a state of {N} x {P}")
+    nr, lpc = (4, 4) if N <= 16 else (4, 8) if N <= 32 else (4, 16) if N <= 64 else (8, 16) if N <= 128 else (16, 16)
+    cols = 256 // lpc
+    return -(-P // cols) * 256 * nr
+
+
 def ssm_scan(u, proj, dt_off, dt_bias, a_log, d_skip, state, meta, out, heads, groups, N, P):
     """The state-space walk of every sequence of the step: u f32 [T, heads P + 2 groups N] (x, B, C as the
     convolution left them), the step sizes' pre-activations in columns [dt_off, + heads) of proj (f32 [T, ld]);
     dt = softplus(. + dt_bias), S <- exp(-exp(a_log) dt) S + dt B x^T, out = S^T C + d_skip x; state f32
-    [slots, heads, N, P] advanced in place, out f32 [T, heads P]."""
+    [slots, heads, ssm_state_floats(N, P)] advanced in place (zeros: an empty state), out f32 [T, heads P]."""
     T = u.shape[0]
     _check(u, "u", torch.float32, (T, heads * P + 2 * groups * N))
     _check(proj, "proj", torch.float32, (T, None))
     for t, name in ((dt_bias, "dt_bias"), (a_log, "A_log"), (d_skip, "D")):
         _check(t, name, torch.float32, (heads,))
-    _check(state, "state", torch.float32, (None, heads, N, P))
+    _check(state, "state", torch.float32, (None, heads, ssm_state_floats(N, P)))
     _check(out, "out", torch.float32, (T, heads * P))
     _check(meta.seq_starts, "seq_starts", torch.int32, (meta.num_seqs + 1,))
     _check(meta.slots, "slots", torch.int32, (meta.num_seqs,))
@@ -59,7 +70,7 @@ def ssm_scan(u, proj, dt_off, dt_bias, a_log, d_skip, state, meta, out, heads, g
         raise BackendError(f"state-space walk: {heads} heads in {groups} groups, a state of {N} rows")
     lib.call("recurrent", "hb_ssm_scan", u.data_ptr(), u.shape[1], proj.data_ptr(), proj.shape[1], int(dt_off),
              dt_bias.data_ptr(), a_log.data_ptr(), d_skip.data_ptr(), state.data_ptr(), meta.seq_starts.data_ptr(),
-             meta.slots.data_ptr(), out.data_ptr(), meta.num_seqs, heads, groups, N, P, _stream())
+             meta.slots.data_ptr(), out.data_ptr(), meta.num_seqs, heads, groups, N, P, state.shape[2], _stream())
 
 
 def gated_group_norm(o, proj, z_off, weight, out, parts, eps):

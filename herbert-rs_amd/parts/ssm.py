@@ -79,7 +79,8 @@ class StateSpace(Part):
                 n["o"]: TensorNeed((W, self.inner))}
 
     def cache_need(self):
-        needs = [StateNeed((self.heads, self.N, self.P), torch.float32)]
+        # (the walk's kernel lays a head's matrix out as its threads hold it)
+        needs = [StateNeed((self.heads, recurrent.ssm_state_floats(self.N, self.P)), torch.float32)]
         if self.taps > 1:
             needs.append(StateNeed((self.taps - 1, self.channels), torch.float32))
         return tuple(needs)

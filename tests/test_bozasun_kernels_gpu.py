@@ -180,7 +180,7 @@ def test_state_space_layer_whole_in_portions_and_token_by_token(heads, P, N, gro
     cut = projs[0].clone()
     cut[0] = 0.0
     assert float((reference(cut)[1][-1] - refs[0][1][-1]).abs().max()) > 1e-3
-    needs = {0: (StateNeed((heads, N, P)), StateNeed((max(K - 1, 1), C)))}
+    needs = {0: (StateNeed((heads, recurrent.ssm_state_floats(N, P))), StateNeed((max(K - 1, 1), C)))}
     cache = Cache(needs, 64 * 8, 4096, torch.float32, DEV, max_slots=4)
     state, conv_state = cache.state_views(0)
     section = 256
