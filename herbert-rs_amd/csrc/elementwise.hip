@@ -1156,7 +1156,7 @@ extern "C" int hb_gate_heads(const void* attn, int dtype, const float* gate_rows
 //     g = gelu_tanh(W_gate x) * e;   y = W_proj g;   x <- x + y / sqrt(mean(y^2) + eps) * w
 // x f32 [T, H] in place; W_gate [D, H], the table, and W_proj transposed [D, H] in one storage type; all arithmetic
 // float32. Three kernels, each of which fills the chip for a few tokens as for thousands:
-//   gate: a workgroup takes SIDE_TOKENS tokens and 4 x RW rows of W_gate; a wave takes RW of them, its lanes
+//   gate: a workgroup takes SIDE_TOKENS tokens and 4 x RW rows of W_gate (RW = 4; eight rows a wave were no faster); a wave takes RW of them, its lanes
 //     share a row's columns (whole lines of the matrix), every x is read once for the wave's RW rows; the sums
 //     over the lanes run in a fixed order; g f32 [T, D]; a step of few tokens gives a row to a whole workgroup;
 //   proj: a workgroup takes SIDE_TOKENS tokens (their g in LDS) and 64 columns of y; a lane takes a column,
@@ -1167,7 +1167,8 @@ extern "C" int hb_gate_heads(const void* attn, int dtype, const float* gate_rows
 template <class TW, int RW>
 __global__ void __launch_bounds__(256)
 token_gate_kernel(const float* __restrict__ x, const int* __restrict__ tokens, const TW* __restrict__ table,
-                  int table_ld, int col0, const TW* __restrict__ w_gate, float* __restrict__ g, int T, int H, int D) {
+                  int table_ld, int col0, const TW* __restrict__ w_gate, float* __restrict__ g, bf16* __restrict__ g16,
+                  int T, int H, int D) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int t0 = blockIdx.y * SIDE_TOKENS;
     const int j0 = (blockIdx.x * 4 + wave) * RW;
@@ -1197,7 +1198,9 @@ token_gate_kernel(const float* __restrict__ x, const int* __restrict__ tokens, c
             const float z = hb_wave_sum(acc[r][k]);
             if (lane == 0 && j0 + r < D && t0 + k < T) {
                 const float gelu = 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
-                g[(size_t)(t0 + k) * D + j0 + r] = gelu * hb_to_float(table[(size_t)tokens[t0 + k] * table_ld + col0 + j0 + r]);
+                const float out = gelu * hb_to_float(table[(size_t)tokens[t0 + k] * table_ld + col0 + j0 + r]);
+                if (g16) g16[(size_t)(t0 + k) * D + j0 + r] = hb_from_float<bf16>(out);       // (for a product on the matrix cores)
+                else g[(size_t)(t0 + k) * D + j0 + r] = out;
             }
         }
 }
@@ -1297,10 +1300,19 @@ add_normed_kernel(float* __restrict__ x, const float* __restrict__ y, const floa
     for (int c = threadIdx.x; c < H; c += 256) x[row + c] += y[row + c] * inv * w[c];
 }
 
-// g f32 [T, D] and y f32 [T, H] are the caller's scratch.
+// g f32 [T, D] and y f32 [T, H] are the caller's scratch. stage 1: all three kernels. stage 0: the gate alone,
+// which leaves g as bfloat16 in g16 [T, D] if that is given (many tokens only): the caller's own product makes y
+// from it; stage 2: the norm and the sum alone, from the caller's y.
 extern "C" int hb_token_side(float* x, const int* tokens, const void* table, int table_ld, int col0, const void* w_gate,
-                             const void* w_proj_t, int dtype, const float* norm_w, float* g, float* y, int T, int H,
-                             int D, float eps, hipStream_t stream) {
+                             const void* w_proj_t, int dtype, const float* norm_w, float* g, void* g16v, float* y, int T,
+                             int H, int D, float eps, int stage, hipStream_t stream) {
+    bf16* const g16 = (bf16*)g16v;
+    if (stage == 2) {
+        HB_REQUIRE(T > 0 && H > 0, "token input: empty input");
+        add_normed_kernel<<<T, 256, 0, stream>>>(x, y, norm_w, H, eps);
+        HB_CHECK_LAUNCH("token_add_normed");
+        return 0;
+    }
     HB_REQUIRE(T > 0 && H > 0 && D > 0, "token input: empty input");
     HB_REQUIRE(col0 >= 0 && col0 + D <= table_ld, "token input: the layer's columns lie outside the table's rows");
     const size_t lds = ((size_t)SIDE_TOKENS * D + 3 * SIDE_TOKENS * 64) * sizeof(float);
@@ -1308,16 +1320,18 @@ extern "C" int hb_token_side(float* x, const int* tokens, const void* table, int
     const int tiles = (T + SIDE_TOKENS - 1) / SIDE_TOKENS;
     HB_REQUIRE(tiles <= 65535, "token input: too many tokens for the grid");
     const bool many = T > 64;          // (few tokens: a row a workgroup, so that the gate's rows are spread over more waves)
+    HB_REQUIRE(g16 == nullptr || (many && stage == 0), "token input: bfloat16 gates are for many tokens and a product of the caller's");
     HB_REQUIRE(D <= 65535, "token input: too many gates for the grid");
 #define HB_SIDE(TW)                                                                                                   \
     do {                                                                                                              \
         if (many)                                                                                                     \
             token_gate_kernel<TW, 4><<<dim3((D + 15) / 16, tiles), 256, 0, stream>>>(                                  \
-                x, tokens, (const TW*)table, table_ld, col0, (const TW*)w_gate, g, T, H, D);                          \
+                x, tokens, (const TW*)table, table_ld, col0, (const TW*)w_gate, g, g16, T, H, D);                     \
         else                                                                                                          \
             token_gate_few_kernel<TW><<<dim3(D, tiles), 256, 0, stream>>>(                                             \
                 x, tokens, (const TW*)table, table_ld, col0, (const TW*)w_gate, g, T, H, D);                          \
         HB_CHECK_LAUNCH("token_gate");                                                                                \
+        if (stage != 1) break;                                                                                        \
         token_proj_kernel<TW><<<dim3((H + 63) / 64, tiles), 256, lds, stream>>>(g, (const TW*)w_proj_t, y, T, H, D);   \
         HB_CHECK_LAUNCH("token_proj");                                                                                \
     } while (0)
@@ -1325,6 +1339,7 @@ extern "C" int hb_token_side(float* x, const int* tokens, const void* table, int
     else if (dtype == HB_BF16) HB_SIDE(bf16);
     else HB_REQUIRE(false, "token input: unknown dtype %d", dtype);
 #undef HB_SIDE
+    if (stage != 1) return 0;
     add_normed_kernel<<<T, 256, 0, stream>>>(x, y, norm_w, H, eps);
     HB_CHECK_LAUNCH("token_add_normed");
     return 0;

@@ -808,23 +808,25 @@ extern "C" int hb_ssm_scan(const float* u, int ldu, const float* proj, int ld, i
 // ------------------------------------------------- gate, then a norm in groups: what leaves the state-space walk
 // v = o silu(z); y = v / sqrt(mean over the group of v^2 + eps) * w: a row of `width` is cut into `parts` equal
 // groups, each normed by its own root mean square; w [width]; z: columns [z_off, + width) of proj's rows.
-// One wave a (token, group).
+// One workgroup a (token, group): a wave for groups of up to 256 channels, four waves beyond; the sum of squares
+// runs in a fixed order.
 template <class TOut>
-__global__ void __launch_bounds__(HB_WAVE)
+__global__ void __launch_bounds__(256)
 gated_group_norm_kernel(const float* __restrict__ o, const float* __restrict__ proj, int ld, int z_off,
                         const float* __restrict__ w, TOut* __restrict__ y, int width, int parts, float eps) {
-    const int t = blockIdx.x, part = blockIdx.y, lane = threadIdx.x;
+    __shared__ float red[16];
+    const int t = blockIdx.x, part = blockIdx.y, tid = threadIdx.x, nt = blockDim.x;
     const int len = width / parts, c0 = part * len;
     const float* in = o + (size_t)t * width + c0;
     const float* gate = proj + (size_t)t * ld + z_off + c0;
     float ss = 0.f;
-    for (int d = lane; d < len; d += HB_WAVE) {
+    for (int d = tid; d < len; d += nt) {
         const float v = in[d] * hb_silu(gate[d]);
         ss = fmaf(v, v, ss);
     }
-    ss = hb_wave_sum(ss);
+    ss = hb_block_sum(ss, red);
     const float inv = 1.0f / sqrtf(ss / (float)len + eps);
-    for (int d = lane; d < len; d += HB_WAVE)
+    for (int d = tid; d < len; d += nt)
         y[(size_t)t * width + c0 + d] = hb_from_float<TOut>(in[d] * hb_silu(gate[d]) * inv * w[c0 + d]);
 }
 
@@ -833,10 +835,11 @@ extern "C" int hb_gated_group_norm(const float* o, const float* proj, int ld, in
     HB_REQUIRE(T > 0 && width > 0 && parts > 0 && width % parts == 0 && parts <= 65535,
                "gated norm in groups: %d columns in %d groups", width, parts);
     HB_REQUIRE(z_off >= 0 && z_off + width <= ld, "gated norm in groups: the gate's columns lie outside the rows");
+    const int threads = width / parts > 256 ? 256 : HB_WAVE;
     if (y_dtype == HB_F32)
-        gated_group_norm_kernel<float><<<dim3(T, parts), HB_WAVE, 0, stream>>>(o, proj, ld, z_off, w, (float*)y, width, parts, eps);
+        gated_group_norm_kernel<float><<<dim3(T, parts), threads, 0, stream>>>(o, proj, ld, z_off, w, (float*)y, width, parts, eps);
     else if (y_dtype == HB_BF16)
-        gated_group_norm_kernel<bf16><<<dim3(T, parts), HB_WAVE, 0, stream>>>(o, proj, ld, z_off, w, (bf16*)y, width, parts, eps);
+        gated_group_norm_kernel<bf16><<<dim3(T, parts), threads, 0, stream>>>(o, proj, ld, z_off, w, (bf16*)y, width, parts, eps);
     else
         HB_REQUIRE(false, "gated norm in groups: unknown output dtype %d", y_dtype);
     HB_CHECK_LAUNCH("gated_group_norm");

@@ -30,7 +30,7 @@ SIGNATURES = {
         "hb_filter_norm_rotate_write": [_P, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P,
                                         _I, _I, _I, _I, _I, _I, _I, _F, _I, _P, _I, _P],
         "hb_add_bias": [_P, _P, _I, _I, _P],
-        "hb_token_side": [_P, _P, _P, _I, _I, _P, _P, _I, _P, _P, _P, _I, _I, _I, _F, _P],
+        "hb_token_side": [_P, _P, _P, _I, _I, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _F, _I, _P],
         "hb_gate_heads": [_P, _I, _P, _I, _I, _P, _I, _I, _I, _I, _P],
         "hb_fill_u32": [_P, _U32, _SZ, _P],
         "hb_layernorm": [_P, _P, _F, _P, _P, _I, _P, _I, _I, _F, _P],

@@ -579,10 +579,19 @@ def add_bias(x, bias):
     lib.call("elementwise", "hb_add_bias", x.data_ptr(), bias.data_ptr(), T, H, _stream())
 
 
-def token_side(x, token_ids, table, col0, w_gate, w_proj_t, norm_w, eps, g, y):
+TOKEN_SIDE_FEW = 64      # up to so many tokens the gate's rows take a workgroup each
+
+
+def token_side(x, token_ids, table, col0, w_gate, w_proj_t, norm_w, eps, g, y, stage=1, g16=None):
     """x += rmsnorm(W_proj (gelu_tanh(W_gate x) * table[token, col0 : col0 + D])) * norm_w, row by row and in
     place: x f32 [T, H], token_ids int32 [T], table [V, ld], W_gate [D, H], W_proj transposed [D, H] (one dtype),
-    norm_w f32 [H]; g f32 [T, D] and y f32 [T, H] are scratch."""
+    norm_w f32 [H]; g f32 [T, D] and y f32 [T, H] are scratch. stage 0: the gate alone (more than TOKEN_SIDE_FEW
+    tokens: into g16 bf16 [T, D] if that is given, for a product of the caller's that makes y); stage 2: the norm
+    and the sum alone, from y."""
+    if g16 is not None:
+        _check(g16, "g16", torch.bfloat16, (x.shape[0], w_gate.shape[0]))
+        if stage != 0 or x.shape[0] <= TOKEN_SIDE_FEW:
+            raise BackendError("token input: bfloat16 gates are for many tokens and a product of the caller's")
     T, H = x.shape
     D = w_gate.shape[0]
     _check(x, "x", torch.float32, (T, H))
@@ -597,7 +606,7 @@ def token_side(x, token_ids, table, col0, w_gate, w_proj_t, norm_w, eps, g, y):
         raise BackendError("token input: the layer's columns lie outside the table's rows")
     lib.call("elementwise", "hb_token_side", x.data_ptr(), token_ids.data_ptr(), table.data_ptr(), table.shape[1],
              int(col0), w_gate.data_ptr(), w_proj_t.data_ptr(), dtype_code(w_gate), norm_w.data_ptr(), g.data_ptr(),
-             y.data_ptr(), T, H, D, float(eps), _stream())
+             _ptr(g16), y.data_ptr(), T, H, D, float(eps), int(stage), _stream())
 
 
 def gate_heads(attn, gate_rows, g_off, out, nq, hd, vdim):

@@ -21,7 +21,7 @@ from .delta import _rate_init, _taps_init
 from .linear import Linear
 from .registry import register
 
-SECTION = 256        # channels of the filter that one wave takes
+SECTION, SECTION_FEW = 256, 64        # channels of the filter that one wave takes; where the step has few tokens
 
 
 def _skip_init(shape, gen, device, std, norm_std):
@@ -104,7 +104,8 @@ class StateSpace(Part):
         self.proj.forward(y, proj)
         u = rt.buffer("ssm_xbc", (T, C), torch.float32)
         conv_state = views[1] if self.taps > 1 else rt.buffer("ssm_no_conv", (1, 1, C), torch.float32)
-        recurrent.conv_silu(proj, self.conv_w, conv_state, ctx.meta, u, 0, 1, 0, 1.0, 0.0, -(-C // SECTION), SECTION,
+        section = SECTION if T > 64 else SECTION_FEW       # (few tokens: more, shorter waves)
+        recurrent.conv_silu(proj, self.conv_w, conv_state, ctx.meta, u, 0, 1, 0, 1.0, 0.0, -(-C // section), section,
                             col0=self.inner, bias=self.conv_b)
         walked = rt.buffer("ssm_y", (T, self.inner), torch.float32)
         recurrent.ssm_scan(u, proj, self.inner + C, self.dt_bias, self.a_log, self.d_skip, views[0], ctx.meta, walked,

@@ -6,8 +6,9 @@ e = that token's row for this layer (columns [i dim, (i + 1) dim) of the table):
     g = gelu_tanh(W_gate x) * e;   y = W_proj g;   x <- x + y / sqrt(mean(y^2) + eps) * w
 
 The gate reads the residual stream x itself, not a normed copy of it. Three small kernels do it (the gate, the
-second product, the norm with the sum), in float32 arithmetic in either mode; the matrices and the table are kept in
-the compute dtype, W_proj transposed so that neighbouring threads read neighbouring weights. The table is one
+second product, the norm with the sum), in float32 arithmetic; the matrices and the table are kept in the compute
+dtype, W_proj transposed so that neighbouring threads read neighbouring weights. In bfloat16 mode a step of many
+tokens leaves the gates as bfloat16 and takes the second product to the matrix cores (float32 sums). The table is one
 tensor for all layers and is kept on the GPU once.
 """
 import torch
@@ -15,6 +16,7 @@ import torch
 from ..kernels import ops
 from ..weights import TensorNeed
 from .base import Part
+from .linear import Linear
 from .registry import register
 
 
@@ -41,12 +43,23 @@ class GatedTableInput(Part):
     def load(self, tensors, rt):
         n = self.names
         self.table = rt.shared_weight(n["table"], tensors[n["table"]])
-        self.gate, self.proj_t = rt.weight(tensors[n["gate"]]), rt.weight(tensors[n["proj"]]).t().contiguous()
+        proj = rt.weight(tensors[n["proj"]])
+        self.gate, self.proj_t = rt.weight(tensors[n["gate"]]), proj.t().contiguous()
+        # bfloat16, many tokens, sizes the matrix cores take: the second product is one of theirs
+        self.proj = None
+        if rt.dtype == torch.bfloat16 and self.dim % 32 == 0 and self.hidden_size % 16 == 0:
+            self.proj = Linear(proj, scratch=rt.scratch)
         self.norm_w = rt.weight(tensors[n["norm"]], matrix=False)
 
     def forward(self, ctx, x):
         T = x.shape[0]
         g = ctx.rt.buffer("token_input_gates", (T, self.dim), torch.float32)
         y = ctx.rt.buffer("token_input_rows", (T, self.hidden_size), torch.float32)
-        ops.token_side(x, ctx.meta.token_ids, self.table, self.layer * self.dim, self.gate, self.proj_t, self.norm_w,
-                       self.eps, g, y)
+        args = (x, ctx.meta.token_ids, self.table, self.layer * self.dim, self.gate, self.proj_t, self.norm_w, self.eps, g, y)
+        if self.proj is not None and T > ops.TOKEN_SIDE_FEW:
+            g16 = ctx.rt.buffer("token_input_gates16", (T, self.dim), torch.bfloat16)
+            ops.token_side(*args, stage=0, g16=g16)
+            self.proj.forward(g16, y)
+            ops.token_side(*args, stage=2)
+            return
+        ops.token_side(*args)
