@@ -209,8 +209,8 @@ def mefatar_configs(size):
 def bozasun_configs(size):
     """(Bozasun config dict, Vipalorn config dict) of one size: of every four layers two state-space layers (twice
     the model's width inside, heads of 64 columns, a state of 128 rows, eight groups, four taps), one attention
-    over chunks of 2,048 positions (biases, a norm a head, the whole head rotated at an eighth of the rates, scores
-    capped at 30) and one latent attention with a gate an entry; every layer with experts chosen by softmax scores
+    over chunks of 2,048 positions (biases, a norm a head, the whole head rotated at a quarter of the rates, scores
+    capped at 50) and one latent attention with a gate an entry; every layer with experts chosen by softmax scores
     within two of four groups, a quarter as many identity experts beside them, and a token input of 256; and the
     Vipalorn model of the same width, depth, heads and experts."""
     W, L, H, D, V, rank, rot, E, top, ff, vocab = FAMILY_SIZES[size]
@@ -219,8 +219,8 @@ def bozasun_configs(size):
     space = {"type": "mamba2", "mixer": {"heads": 2 * W // 64, "vdim": 64, "state": 128, "groups": 8, "conv": 4,
                                          "norm_groups": 8}}
     attention = {"type": "attention", "mixer": {"heads": H, "kv_heads": H // 2, "dim": D, "vdim": V, "scale": D ** -0.5,
-                                                "rot": {"dims": D, "base": 500000.0, "scaling": {"factor": 8.0}},
-                                                "mask": {"size": 2048}, "softcap": 30.0}}
+                                                "rot": {"dims": D, "base": 1000000.0, "scaling": {"factor": 4.0}},
+                                                "mask": {"size": 2048}, "softcap": 50.0}}
     latent = {"type": "latent_attention", "mixer": {"heads": H, "dim": D, "rot_dim": rot, "vdim": V, "kv_rank": rank,
                                                     "scale": (D + rot) ** -0.5, "rot": {"base": 10000.0, "dims": rot}}}
     layers = [dict((space, attention, space, latent)[i % 4], mlp=mlp) for i in range(L)]

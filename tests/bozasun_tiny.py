@@ -116,9 +116,9 @@ def _s():
 
 def _w():
     # W: the widths of a larger model's layers at a small depth: heads of 128, a state of 128 rows and columns of 64
-    layers = [attention(8, 2, 128, 128, 0.09, rot(128, 500000.0, 8.0), chunk=192, softcap=30.0, mlp=moe(256, 8, 2, identity=4, groups=(4, 2))),
+    layers = [attention(8, 2, 128, 128, 0.09, rot(128, 250000.0, 4.0), chunk=192, softcap=25.0, mlp=moe(256, 8, 2, identity=2, groups=(5, 2))),
               mamba(8, 64, 128, 2, 4, norm_groups=2, mlp=dense(1024)),
-              latent(8, 64, 32, 64, 256, 0.1, 10000.0, mlp=moe(256, 8, 2, identity=4, groups=(4, 2)))]
+              latent(8, 64, 32, 64, 256, 0.1, 10000.0, mlp=moe(256, 8, 2, identity=2, groups=(5, 2)))]
     return model(1024, 512, layers, eps=1e-6, side=64)
 
 
