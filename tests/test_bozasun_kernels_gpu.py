@@ -153,7 +153,8 @@ def test_bias_a_column():
 
 # ---------------------------------------------------------------- the state-space layer
 @pytest.mark.parametrize("heads,P,N,groups,K,parts", [(1, 5, 8, 1, 1, 1), (3, 24, 10, 1, 3, 3), (4, 32, 16, 2, 4, 4), (6, 16, 64, 3, 2, 2),
-                                                      (2, 64, 128, 2, 4, 1), (1, 80, 40, 1, 2, 2), (2, 20, 200, 1, 3, 1)])
+                                                      (2, 64, 128, 2, 4, 1), (1, 80, 40, 1, 2, 2), (2, 20, 200, 1, 3, 1), (2, 12, 24, 1, 2, 1),
+                                                      (8, 80, 16, 2, 3, 1)])
 def test_state_space_layer_whole_in_portions_and_token_by_token(heads, P, N, groups, K, parts):
     """The rows [z | x | B | C | dt] as the projection leaves them: the filter with its bias and silu, the walk with
     decays near one (a long memory) and far below, the gate before the norm in groups."""
@@ -161,7 +162,7 @@ def test_state_space_layer_whole_in_portions_and_token_by_token(heads, P, N, gro
     ld = 2 * inner + 2 * groups * N + heads
     lengths = [41, 3, 18]
     taps, conv_b = 1.0 / K + 0.3 * rand(C, K, seed=5), 0.3 * rand(C, seed=6)
-    a_log = torch.tensor([-6.0, 0.5, -1.0, 0.2, -3.0, 0.0])[:heads]
+    a_log = torch.tensor([-6.0, 0.5, -1.0, 0.2, -3.0, 0.0, -4.0, 0.3])[:heads]
     dt_bias, d_skip, norm_w = 0.3 * rand(heads, seed=7), 1 + 0.3 * rand(heads, seed=8), 1 + 0.2 * rand(inner, seed=9)
     projs = [rand(n, ld, seed=10 + i, scale=1.5) for i, n in enumerate(lengths)]
 
